@@ -1,0 +1,191 @@
+/* qmoe.h -- C ABI of libqmoe_hip.so: GGUF packed-weight linear and packed-expert
+ * MoE step on one AMD Instinct MI355X (gfx950).
+ *
+ * Conventions (they follow the reference's existing native library,
+ * mini_llm/ops/native_packed_cpu.cpp:206-246, loaded by
+ * mini_llm/ops/native_packed_cpu.py:67-77):
+ *   - every function is extern "C", takes plain pointers and sizes, and returns an
+ *     int status: 0 = success, nonzero = error; on error no kernel has touched the
+ *     output.  qmoe_last_error() returns a thread-local message for the last
+ *     nonzero status on the calling thread.
+ *   - every pointer named w/gate/up/down/x/y/out/logits/... is DEVICE memory on the
+ *     current HIP device unless its comment says "host".  The caller owns all
+ *     buffers; the library keeps no pointer after the call's work has drained from
+ *     `stream`.  Weights and inputs are never written.
+ *   - work is enqueued asynchronously on `stream` (a hipStream_t passed as void*;
+ *     NULL = the null stream).  No call synchronises the device or allocates
+ *     device memory; calls that need scratch take a caller-provided workspace.
+ *   - packed matrices are row-major [N, K] GGUF blocks packed along K; expert banks
+ *     are [E, N, K] with a byte stride between experts
+ *     (mini_llm/ops/quantized_weight.py:85-99).
+ */
+#ifndef QMOE_H
+#define QMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QMOE_ABI_VERSION 1
+
+/* Packed formats.  Ids 0..5 are the reference's (_FORMAT_ID,
+ * mini_llm/ops/quantized_linear.py:34 and native_packed_cpu.cpp:12).  BF16 has no
+ * packed id in the reference (it is decoded as a dense tensor,
+ * mini_llm/external/gguf_tensor.py:30-51); id 100 is this library's extension. */
+enum {
+    QMOE_FMT_Q8_0 = 0,
+    QMOE_FMT_Q4_0 = 1,
+    QMOE_FMT_Q4_K = 2,
+    QMOE_FMT_Q3_K = 3, /* recognised, not implemented: QMOE_EUNSUPPORTED */
+    QMOE_FMT_Q5_K = 4,
+    QMOE_FMT_Q6_K = 5,
+    QMOE_FMT_BF16 = 100
+};
+
+/* Activation / output element types. */
+enum { QMOE_DT_F32 = 0, QMOE_DT_F16 = 1, QMOE_DT_BF16 = 2 };
+
+/* Status codes. */
+enum {
+    QMOE_OK = 0,
+    QMOE_EINVAL = 1,       /* null pointer, bad shape, K not a block multiple, ... */
+    QMOE_EUNSUPPORTED = 2, /* format / dtype / size outside what the kernels cover */
+    QMOE_ELAUNCH = 3,      /* HIP reported a launch error */
+    QMOE_EWORKSPACE = 4    /* workspace missing, misaligned or too small */
+};
+
+int qmoe_abi_version(void);
+const char* qmoe_last_error(void);
+
+/* Elements and bytes per block of a format (BLOCK_FORMATS,
+ * mini_llm/ops/quantized_weight.py:24-37). */
+int qmoe_format_info(int fmt, int* block_elems, int* block_bytes);
+
+/* out[n*k] fp32 = dequantised packed matrix; bit-identical to
+ * PackedGGUFWeight.dequantize_reference (mini_llm/ops/quantized_weight.py:151-250)
+ * and, for BF16, to decode_gguf_dense (mini_llm/external/gguf_tensor.py:48-51). */
+int qmoe_dequantize(const void* w, int fmt, int64_t n, int64_t k, float* out, void* stream);
+
+/* y[tokens, n] = x[tokens, k] @ W[n, k]^T with fp32 accumulation; replaces the
+ * device branch of quantized_linear (mini_llm/ops/quantized_linear.py:306-335) and
+ * has the argument order of mylocal_packed_gemv (native_packed_cpu.cpp:208-217)
+ * with element types and a stream added.  x and y are contiguous. */
+int qmoe_linear(const void* w, int fmt, int n, int k,
+                const void* x, int x_dtype, int tokens,
+                void* y, int y_dtype, void* stream);
+
+/* One problem of a batched launch: y = x @ W^T.  Host struct. */
+typedef struct qmoe_linear_problem {
+    const void* w;
+    const void* x;
+    void* y;
+    int fmt, n, k, tokens;
+    int x_dtype, y_dtype;
+} qmoe_linear_problem;
+
+/* Several independent linears enqueued as one launch sequence (e.g. q/k/v of one
+ * layer, which share x); `problems` is a HOST array read before the call returns.
+ * No counterpart in the reference, which launches each projection separately
+ * (mini_llm/external/gguf_projection.py:40-62). */
+int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stream);
+
+/* h[tokens, f] = silu(x @ G^T) * (x @ U^T); gate and up may differ in format.
+ * Replaces the device branch of quantized_swiglu
+ * (mini_llm/ops/quantized_linear.py:338-400). */
+int qmoe_swiglu(const void* gate, int gate_fmt, const void* up, int up_fmt, int f, int k,
+                const void* x, int x_dtype, int tokens,
+                void* h, int h_dtype, void* stream);
+
+/* out[tokens, d_model] = down(swiglu(x)): one packed SwiGLU expert.  Argument
+ * order of mylocal_packed_expert (native_packed_cpu.cpp:219-245).  `workspace` holds
+ * tokens*d_ff fp32 (the stored hidden activation). */
+int qmoe_expert(const void* gate, int gate_fmt, const void* up, int up_fmt,
+                const void* down, int down_fmt, int d_model, int d_ff,
+                const void* x, int x_dtype, int tokens,
+                void* out, int out_dtype, float* workspace, void* stream);
+
+/* Rows of full softmax -> exact top-k (descending logit, lower id on ties, NaN
+ * last) -> optional division by max(selected mass, floor).  weights fp32
+ * [tokens,k], ids int64 [tokens,k].  Replaces expert_topk_forward +
+ * RouterInference's renormalisation (mini_llm/ops/router.py:21-43,
+ * mini_llm/ops/router_inference.py:47-61) and the single-row kernel
+ * normalized_topk (mini_llm/ops/router_decode.py:27-95).  n <= 4096, k <= 32. */
+int qmoe_router_topk(const float* logits, int tokens, int n, int k, float floor_value,
+                     int renormalize, float* weights, int64_t* ids, void* stream);
+
+/* A bank of E SwiGLU experts stored as three packed tensors [E,F,D], [E,F,D],
+ * [E,D,F] (Qwen3NextGGUFIndex.expert_weights,
+ * mini_llm/external/qwen3next_gguf.py:153-169).  A fused gate_up tensor [E,2F,D] is
+ * described by up = gate + F rows and both strides = 2F rows.  Host struct. */
+typedef struct qmoe_expert_bank {
+    const void* gate;
+    const void* up;
+    const void* down;
+    int64_t gate_stride, up_stride, down_stride; /* bytes between experts */
+    int gate_fmt, up_fmt, down_fmt;
+    int n_experts, d_model, d_ff;
+} qmoe_expert_bank;
+
+/* Single token, E selected experts given as a DEVICE table of E rows of three
+ * device pointers (gate, up, down) in the order they are to be summed.
+ * out[d] = sum over rows, sequentially from zero, of
+ *          fp32(down_e(fp32 swiglu_e(x))[d] * routes[slot_e * route_stride])
+ * with the product stored before each add (no FMA, no tree).  slots is a DEVICE
+ * int32 array of E route positions or NULL for slot_e = e.  Replaces
+ * grouped_quantized_experts_forward
+ * (mini_llm/ops/grouped_quantized_experts.py:159-217).  workspace: fp32
+ * E*d_ff + E*d_model elements. */
+int qmoe_grouped_decode(const float* x, const void* const* table, int n_rows,
+                        int gate_fmt, int up_fmt, int down_fmt, int d_model, int d_ff,
+                        const float* routes, int64_t route_stride, const int32_t* slots,
+                        float* out, float* workspace, void* stream);
+
+/* Arguments of one MoE step over T tokens.  Host struct. */
+typedef struct qmoe_moe_args {
+    const void* hidden;     /* [T, d_model], hidden_dtype */
+    int hidden_dtype;
+    int tokens;
+    int top_k;
+    /* routing input: either logits (router runs on device) or precomputed
+     * weights + ids (both device); logits wins when non-NULL. */
+    const float* logits;    /* [T, n_experts] fp32 or NULL */
+    float floor_value;      /* renormalisation floor, 2^-14 for Qwen3-Next */
+    int renormalize;
+    const float* in_weights;  /* [T, k] fp32, used when logits == NULL */
+    const int64_t* in_ids;    /* [T, k] int64, used when logits == NULL */
+    qmoe_expert_bank bank;
+    /* shared expert (all NULL = none): gate/up [d_ff_shared, d_model], down
+     * [d_model, d_ff_shared]; shared_gate fp32 [d_model] or NULL (= ungated). */
+    const void* shared_gate_w;
+    const void* shared_up_w;
+    const void* shared_down_w;
+    int shared_gate_fmt, shared_up_fmt, shared_down_fmt;
+    int d_ff_shared;
+    const float* shared_gate;
+    void* out;              /* [T, d_model], out_dtype */
+    int out_dtype;
+    float* out_weights;     /* optional [T, k] fp32: routing weights used */
+    int64_t* out_ids;       /* optional [T, k] int64: selected experts */
+} qmoe_moe_args;
+
+/* Bytes of workspace qmoe_moe_forward needs for these sizes (256-byte aligned). */
+size_t qmoe_moe_workspace_bytes(int tokens, int top_k, int n_experts, int d_model,
+                                int d_ff, int d_ff_shared);
+
+/* routed + shared * sigmoid(hidden . shared_gate): router (optional), device-side
+ * token->expert compaction, packed experts, ordered weighted combine (ascending
+ * expert id per token, product stored then added), shared expert.  Replaces
+ * Qwen3NextMoEInference.forward (mini_llm/external/qwen3next_moe.py:129-147) with
+ * ExpertsInference.forward's general path (mini_llm/ops/experts_inference.py:290-310)
+ * and RoutingPlan.from_router_outputs (mini_llm/ops/routing_plan.py:52-118) inside;
+ * there is no host round trip. */
+int qmoe_moe_forward(const qmoe_moe_args* args, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QMOE_H */

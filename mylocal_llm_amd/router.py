@@ -1,0 +1,101 @@
+"""Expert router on the device: full softmax, exact top-k, optional renormalisation.
+
+Same entry points as the reference: ``expert_topk_forward`` (mini_llm/ops/router.py:21-43),
+``RouterInference`` (mini_llm/ops/router_inference.py:10-61) and ``try_normalized_topk``
+(mini_llm/ops/router_decode.py:247-273).  Selection order is descending logit, lower expert
+id on exact ties, NaN last (router_decode.py:19-26); ids are int64.
+"""
+import math
+
+import numpy as np
+import torch
+
+from . import _lib
+from .quantized_linear import _ptr, _stream
+
+_MAX_EXPERTS = 4096
+_MAX_K = 32
+
+
+def _topk(logits2d, k, floor, renormalize):
+    t, n = logits2d.shape
+    weights = torch.empty((t, k), dtype=torch.float32, device=logits2d.device)
+    ids = torch.empty((t, k), dtype=torch.int64, device=logits2d.device)
+    if t:
+        with torch.cuda.device(logits2d.device):
+            rc = _lib.load().qmoe_router_topk(_ptr(logits2d), t, n, k, float(floor), int(renormalize),
+                                              _ptr(weights), _ptr(ids), _stream())
+        _lib.check(rc, "Router top-k")
+    return weights, ids
+
+
+def expert_topk_forward(logits, k, output_dtype=None, return_cache=True):
+    """Full-expert softmax followed by top-k selection, without renormalisation."""
+    if not isinstance(logits, torch.Tensor) or not logits.is_cuda:
+        raise TypeError("router logits must be a CUDA torch.Tensor")
+    if logits.ndim < 1 or not (1 <= int(k) <= int(logits.shape[-1])):
+        raise ValueError("expert router expects 1 <= k <= n_experts")
+    n = logits.shape[-1]
+    if n > _MAX_EXPERTS or int(k) > _MAX_K:
+        raise NotImplementedError("router kernel covers at most 4096 experts and k <= 32")
+    work = logits.to(torch.float32).contiguous().reshape(-1, n)
+    weights, ids = _topk(work, int(k), 1.0, False)
+    shape = tuple(logits.shape[:-1]) + (int(k),)
+    weights = weights.reshape(shape)
+    if output_dtype is not None and output_dtype in (torch.float16, torch.bfloat16):
+        weights = weights.to(output_dtype)
+    return weights, ids.reshape(shape), None
+
+
+def try_normalized_topk(logits, k, normalization_floor):
+    """Weights/ids for fp32 logits, or None for metadata the kernel does not cover."""
+    tiny, big = float(np.finfo(np.float32).tiny), float(np.finfo(np.float32).max)
+    if (not isinstance(logits, torch.Tensor) or not logits.is_cuda
+            or logits.dtype != torch.float32 or not logits.is_contiguous()
+            or logits.ndim < 1 or not 1 <= logits.shape[-1] <= _MAX_EXPERTS
+            or not 1 <= k <= min(_MAX_K, logits.shape[-1])
+            or not tiny <= normalization_floor <= big):
+        return None
+    n = logits.shape[-1]
+    weights, ids = _topk(logits.reshape(-1, n), int(k), normalization_floor, True)
+    shape = tuple(logits.shape[:-1]) + (int(k),)
+    return weights.reshape(shape), ids.reshape(shape)
+
+
+class RouterInference:
+    """Full-softmax-then-top-k router; optional inference-only renormalisation."""
+
+    def __init__(self, d_model, n_experts, k, dtype="float32", *,
+                 renormalize_selected=False, normalization_floor=1e-30):
+        self.d_model = d_model
+        self.n_experts = n_experts
+        if not (1 <= int(k) <= int(n_experts)):
+            raise ValueError("expert router expects 1 <= k <= n_experts")
+        self.k = int(k)
+        if not isinstance(renormalize_selected, bool):
+            raise TypeError("renormalize_selected must be bool")
+        if not math.isfinite(normalization_floor) or normalization_floor <= 0:
+            raise ValueError("normalization_floor must be finite and positive")
+        self.renormalize_selected = renormalize_selected
+        self.normalization_floor = float(normalization_floor)
+        self.W_router = None
+        self.b_router = None
+
+    def route_logits(self, logits):
+        """Selection and weights from precomputed logits [B, T, E] (or [T, E])."""
+        if self.renormalize_selected:
+            floor = max(self.normalization_floor, float(np.finfo(np.float32).tiny))
+            decoded = try_normalized_topk(logits.to(torch.float32).contiguous(), self.k, floor)
+            if decoded is None:
+                raise NotImplementedError("router kernel covers at most 4096 experts and k <= 32")
+            return decoded
+        weights, ids, _ = expert_topk_forward(logits, self.k, return_cache=False)
+        return weights, ids
+
+    def forward(self, x):
+        batch_size, seq_len, _ = x.shape
+        x2 = x.reshape(batch_size * seq_len, self.d_model)
+        logits = x2 @ self.W_router + self.b_router
+        logits = logits.reshape(batch_size, seq_len, self.n_experts)
+        weights, ids = self.route_logits(logits)
+        return weights.to(x.dtype), ids

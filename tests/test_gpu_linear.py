@@ -1,0 +1,194 @@
+"""GPU linear / SwiGLU / expert parity through the C ABI against the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import native, reference_np as R
+from mylocal_llm_amd import synthetic
+from mylocal_llm_amd.quantized_weight import PackedGGUFWeight
+from mylocal_llm_amd.quantized_linear import (
+    PackedExpertFFNInference, quantized_linear, quantized_linear_batch, quantized_swiglu,
+)
+from gpu_util import BF16_MAX_ABS, REL_L2, announce, rel_l2, triple, upload
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+RV = np.load(os.path.join(GOLDEN, "ref_native_vectors.npz"))
+FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K", "BF16"]
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 16, 64])
+def test_linear_matches_oracle(cuda, fmt, m):
+    announce("linear", fmt, "M", m)
+    w = synthetic.packed_weight(fmt, (96, 1024), 106)
+    x = synthetic.activations((m, 1024), 103)
+    want = R.linear(x, *triple(w))
+    got = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    assert got.shape == (m, 96) and got.dtype == np.float32
+    assert rel_l2(got, want) <= 2e-6 <= REL_L2
+    np.testing.assert_allclose(got, native.c_linear(x, *triple(w)), rtol=2e-5, atol=2e-5 * np.abs(want).max())
+
+
+def test_config0_single_q8_0_matrix_batch1(cuda):
+    # benchmark configuration 0: 2048 x 2048 Q8_0, fp32 [1, 2048]
+    w = synthetic.packed_weight("Q8_0", (2048, 2048), 106)
+    x = synthetic.activations((1, 2048), 103)
+    want = R.linear(x, *triple(w))
+    got = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    assert rel_l2(got, want) <= 2e-6
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"])
+def test_linear_reference_native_vectors(cuda, fmt):
+    blocks, x, y = RV[fmt + "_blocks"], RV[fmt + "_x"], RV[fmt + "_gemv"]
+    w = PackedGGUFWeight(blocks, (y.shape[1], x.shape[1]), fmt)
+    got = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    np.testing.assert_allclose(got, y, rtol=3e-5, atol=2e-4 * max(np.abs(y).max(), 1))
+
+
+@pytest.mark.parametrize("rows", [65536, 151936])
+@pytest.mark.parametrize("tokens", [1, 2])
+def test_large_output_projection_exact(cuda, rows, tokens):
+    # every partial sum is exactly representable, so any summation order must give equality
+    announce("linear large N", rows, tokens)
+    q = np.broadcast_to((np.arange(rows, dtype=np.int64) % 15 - 7).astype(np.int8)[:, None], (rows, 32)).copy()
+    raw = np.concatenate((np.full((rows, 1), .125, "<f2").view(np.uint8), q.view(np.uint8)), axis=1).reshape(-1)
+    w = PackedGGUFWeight(raw, (rows, 32), "Q8_0")
+    hidden = np.stack([(np.arange(32, dtype=np.float32) + t) / 32 for t in range(tokens)])
+    expected = hidden.sum(axis=1, keepdims=True) * (q[:, 0].astype(np.float32) * .125)[None]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        got = quantized_linear(torch.from_numpy(hidden).to(cuda), upload(w, cuda))
+    stream.synchronize()
+    np.testing.assert_array_equal(got.cpu().numpy(), expected)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, BF16_MAX_ABS)])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+def test_linear_low_precision_activations(cuda, dtype, tol, fmt):
+    announce("linear lowp", fmt, dtype)
+    w = synthetic.packed_weight(fmt, (64, 512), 7)
+    x = torch.from_numpy(synthetic.activations((3, 512), 5)).to(dtype)
+    # oracle on the exactly representable upcast inputs; output rounded once to the dtype
+    want = R.linear(x.float().numpy(), *triple(w))
+    got = quantized_linear(x.to(cuda), upload(w, cuda))
+    assert got.dtype == dtype
+    want_rounded = torch.from_numpy(want).to(dtype).float().numpy()
+    assert np.abs(got.float().cpu().numpy() - want_rounded).max() <= tol
+    assert rel_l2(got.float().cpu().numpy(), want) <= (5e-3 if dtype == torch.bfloat16 else 1e-3)
+
+
+def test_linear_three_dimensional_input_and_shape_errors(cuda):
+    w = upload(synthetic.packed_weight("Q4_K", (7, 512), 1), cuda)
+    x = torch.from_numpy(synthetic.activations((2, 3, 512), 2)).to(cuda)
+    y = quantized_linear(x, w)
+    assert y.shape == (2, 3, 7)
+    np.testing.assert_array_equal(y.reshape(6, 7).cpu().numpy(), quantized_linear(x.reshape(6, 512), w).cpu().numpy())
+    with pytest.raises(ValueError, match="Input K"):
+        quantized_linear(torch.zeros((2, 128), device=cuda), w)
+    with pytest.raises(ValueError, match="Expected x"):
+        quantized_linear(torch.zeros((512,), device=cuda), w)
+    with pytest.raises(ValueError, match="block_k"):
+        quantized_linear(x, w, block_k=128)
+    with pytest.raises(ValueError, match="contiguous"):
+        quantized_linear(torch.zeros((2, 1024), device=cuda)[:, ::2], w)
+    with pytest.raises(TypeError, match="FP16"):
+        quantized_linear(torch.zeros((2, 512), device=cuda, dtype=torch.float64), w)
+    assert quantized_linear(torch.zeros((0, 512), device=cuda), w).shape == (0, 7)
+
+
+def test_linear_inputs_and_weights_are_not_mutated(cuda):
+    w = synthetic.packed_weight("Q6_K", (16, 512), 1)
+    dev = upload(w, cuda)
+    x = torch.from_numpy(synthetic.activations((2, 512), 2)).to(cuda)
+    before = x.clone()
+    quantized_linear(x, dev)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(dev.data.cpu().numpy(), w.data)
+    assert torch.equal(x, before)
+
+
+def test_linear_batch_equals_separate_calls(cuda):
+    ws = [upload(synthetic.packed_weight(f, (n, 512), i), cuda) for i, (f, n) in enumerate([("Q8_0", 64), ("Q6_K", 32), ("Q5_K", 16)])]
+    x = torch.from_numpy(synthetic.activations((2, 512), 9)).to(cuda)
+    outs = quantized_linear_batch([(x, w) for w in ws])
+    for out, w in zip(outs, ws):
+        assert torch.equal(out, quantized_linear(x, w))
+
+
+@pytest.mark.parametrize("gf,uf", [("Q8_0", "Q8_0"), ("Q5_K", "Q4_K"), ("Q6_K", "Q6_K"), ("Q5_K", "Q5_K"), ("BF16", "Q8_0")])
+@pytest.mark.parametrize("m", [1, 3, 16])
+def test_swiglu_fused_matches_oracle_and_unfused(cuda, gf, uf, m):
+    announce("swiglu", gf, uf, m)
+    gate, up = synthetic.packed_weight(gf, (128, 512), 1), synthetic.packed_weight(uf, (128, 512), 2)
+    # scale activations so that gate pre-activations are O(1)
+    x = synthetic.activations((m, 512), 3) * np.float32(2.0)
+    want = R.swiglu(x, triple(gate), triple(up))
+    dg, du = upload(gate, cuda), upload(up, cuda)
+    xd = torch.from_numpy(x).to(cuda)
+    got = quantized_swiglu(xd, dg, du).cpu().numpy()
+    assert rel_l2(got, want) <= 5e-6 <= REL_L2
+    g, u = quantized_linear(xd, dg), quantized_linear(xd, du)
+    unfused = ((g / (1 + torch.exp(-g))) * u).cpu().numpy()
+    np.testing.assert_allclose(got, unfused, rtol=3e-4, atol=2e-4 * np.abs(want).max())
+    with pytest.raises(ValueError, match="gate/up"):
+        quantized_swiglu(xd, dg, upload(synthetic.packed_weight(uf, (64, 512), 2), cuda))
+    with pytest.raises(ValueError, match="K"):
+        quantized_swiglu(torch.zeros((1, 256), device=cuda), dg, du)
+    with pytest.raises(TypeError, match="packed"):
+        quantized_swiglu(xd, dg, object())
+
+
+@pytest.mark.parametrize("fmts", [("Q8_0", "Q8_0", "Q8_0"), ("Q5_K", "Q5_K", "Q6_K"), ("Q6_K", "Q6_K", "Q6_K")])
+@pytest.mark.parametrize("fuse", [True, False])
+def test_packed_expert_matches_oracle(cuda, fmts, fuse):
+    announce("expert", fmts, fuse)
+    d, f = 512, 256
+    gate, up, down = (synthetic.packed_weight(fmts[0], (f, d), 1), synthetic.packed_weight(fmts[1], (f, d), 2),
+                      synthetic.packed_weight(fmts[2], (d, f), 3))
+    x = synthetic.activations((3, d), 4)
+    want = R.expert_ffn(x, triple(gate), triple(up), triple(down))
+    expert = PackedExpertFFNInference(upload(gate, cuda), upload(up, cuda), upload(down, cuda), fuse_gate_up=fuse)
+    got = expert.forward(torch.from_numpy(x).to(cuda)).cpu().numpy()
+    assert rel_l2(got, want) <= 1e-5 <= REL_L2
+    with pytest.raises(ValueError, match="transposed"):
+        PackedExpertFFNInference(expert.gate, expert.up, expert.gate)
+
+
+def test_expert_reference_native_vector(cuda):
+    d = RV["expert_x"].shape[1]
+    f = RV["expert_gate"].shape[0] * 256 // d
+    gate = PackedGGUFWeight(RV["expert_gate"], (f, d), "Q5_K")
+    up = PackedGGUFWeight(RV["expert_up"], (f, d), "Q5_K")
+    down = PackedGGUFWeight(RV["expert_down"], (d, f), "Q6_K")
+    expert = PackedExpertFFNInference(upload(gate, cuda), upload(up, cuda), upload(down, cuda))
+    got = expert.forward(torch.from_numpy(RV["expert_x"]).to(cuda)).cpu().numpy()
+    np.testing.assert_allclose(got, RV["expert_out"], rtol=3e-5, atol=2e-4 * np.abs(RV["expert_out"]).max())
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("shape", [(4096, 4096), (1024, 4096), (4096, 14336)])
+def test_8b_projection_shapes_linearity_and_row_checks(cuda, fmt, shape):
+    """Full-size shapes: spot rows against the oracle plus linearity in x (size-independent)."""
+    announce("linear 8B shape", fmt, shape)
+    n, k = shape
+    w = synthetic.packed_weight(fmt, (n, k), 106)
+    dev = upload(w, cuda)
+    rng = np.random.default_rng(103)
+    x = rng.standard_normal((2, k), dtype=np.float32)
+    xd = torch.from_numpy(x).to(cuda)
+    y = quantized_linear(xd, dev)
+    # linearity: W(a*x0 + b*x1) == a*W x0 + b*W x1 up to fp32 rounding
+    combo = torch.from_numpy((0.5 * x[0] - 0.25 * x[1])[None]).to(cuda)
+    yc = quantized_linear(combo, dev)
+    lin = 0.5 * y[0] - 0.25 * y[1]
+    assert rel_l2(yc[0].cpu().numpy(), lin.cpu().numpy()) <= 1e-5
+    rows = rng.choice(n, 24, replace=False)
+    sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), fmt)
+    want = R.linear(x, *triple(sub))
+    got = y.cpu().numpy()[:, rows]
+    assert rel_l2(got, want) <= 2e-6

@@ -1,0 +1,302 @@
+"""GPU packed-expert MoE step, grouped decode and dispatch/combine against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import reference_np as R
+from mylocal_llm_amd import synthetic
+from mylocal_llm_amd.grouped_quantized_experts import (
+    grouped_quantized_experts_forward, supports_grouped_quantized_experts,
+)
+from mylocal_llm_amd.moe import DevicePackedExpertBank, ExpertsInference, Qwen3NextMoEInference, moe_step
+from mylocal_llm_amd.quantized_linear import PackedExpertFFNInference
+from gpu_util import BF16_MAX_ABS, REL_L2, announce, rel_l2, triple, upload
+
+pytestmark = pytest.mark.gpu
+_FULL = {}
+
+
+def full_layer(fmt, cuda):
+    """512-expert layer of the benchmark shape, built once per format (host + device copies)."""
+    if fmt not in _FULL:
+        e, d, f, fsh = 512, 2048, 512, 2048
+        gate = synthetic.packed_weight(fmt, (e, f, d), 1)
+        up = synthetic.packed_weight(fmt, (e, f, d), 2)
+        down = synthetic.packed_weight(fmt, (e, d, f), 3)
+        shared = (synthetic.packed_weight(fmt, (fsh, d), 4), synthetic.packed_weight(fmt, (fsh, d), 5),
+                  synthetic.packed_weight(fmt, (d, fsh), 6))
+        gate_vec = np.random.default_rng(1).normal(0, .02, d).astype(np.float32)
+        bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+        dshared = tuple(upload(w, cuda) for w in shared)
+        _FULL[fmt] = (gate, up, down, shared, gate_vec, bank, dshared)
+    return _FULL[fmt]
+
+
+def make_layer(e, d, f, fsh, fmts, seed):
+    gate = synthetic.packed_weight(fmts[0], (e, f, d), seed)
+    up = synthetic.packed_weight(fmts[1], (e, f, d), seed + 1)
+    down = synthetic.packed_weight(fmts[2], (e, d, f), seed + 2)
+    shared = (synthetic.packed_weight(fmts[0], (fsh, d), seed + 3), synthetic.packed_weight(fmts[1], (fsh, d), seed + 4),
+              synthetic.packed_weight(fmts[2], (d, fsh), seed + 5))
+    gate_vec = np.random.default_rng(seed + 6).normal(0, .05, d).astype(np.float32)
+    return gate, up, down, shared, gate_vec
+
+
+def oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec):
+    e = gate.shape[0]
+
+    def expert_fn(i, rows):
+        return R.expert_ffn(rows, triple(gate.select_outer(i)), triple(up.select_outer(i)), triple(down.select_outer(i)))
+
+    return R.moe_forward(hidden, logits, k, e, expert_fn, tuple(triple(w) for w in shared), gate_vec)
+
+
+@pytest.mark.parametrize("fmts", [("Q8_0", "Q8_0", "Q8_0"), ("Q6_K", "Q6_K", "Q6_K"), ("Q5_K", "Q5_K", "Q6_K")])
+@pytest.mark.parametrize("tokens", [1, 4, 16, 40])
+def test_moe_step_matches_oracle(cuda, fmts, tokens):
+    announce("moe step", fmts, tokens)
+    e, d, f, fsh, k = 16, 256, 256, 512, 4
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh, fmts, 300)
+    hidden = synthetic.activations((tokens, d), 7, "bf16") * np.float32(4.0)
+    logits = synthetic.router_logits(tokens, e, 9)
+    assert not synthetic.has_topk_ties(logits, k)
+    want, want_w, want_ids = oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    dshared = tuple(upload(w, cuda) for w in shared)
+    hd = torch.from_numpy(hidden).to(cuda)
+    out, w, ids = moe_step(hd, bank, k, logits=torch.from_numpy(logits).to(cuda), shared=dshared,
+                           shared_gate=torch.from_numpy(gate_vec).to(cuda), return_routing=True)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=2e-7)
+    assert rel_l2(out.cpu().numpy(), want) <= 2e-5 <= REL_L2
+    # bf16 hidden states in, bf16 out: same fp32 result rounded once
+    out16 = moe_step(hd.to(torch.bfloat16), bank, k, logits=torch.from_numpy(logits).to(cuda), shared=dshared,
+                     shared_gate=torch.from_numpy(gate_vec).to(cuda))
+    assert out16.dtype == torch.bfloat16
+    scale = max(1.0, float(np.abs(want).max()))
+    assert np.abs(out16.float().cpu().numpy() - want).max() <= BF16_MAX_ABS * scale
+
+
+def test_moe_step_fused_gate_up_bank_and_no_shared(cuda):
+    e, d, f, k = 8, 256, 256, 2
+    gate_up = synthetic.packed_weight("Q8_0", (e, 2 * f, d), 31)
+    down = synthetic.packed_weight("Q8_0", (e, d, f), 32)
+    hidden = synthetic.activations((5, d), 3) * np.float32(4.0)
+    logits = synthetic.router_logits(5, e, 4)
+
+    def expert_fn(i, rows):
+        both = gate_up.select_outer(i)
+        return R.expert_ffn(rows, triple(both.select_rows(0, f)), triple(both.select_rows(f, 2 * f)),
+                            triple(down.select_outer(i)))
+
+    w, ids = R.router_topk(logits, k)
+    want = R.experts_forward(hidden, w, ids, e, expert_fn)
+    bank = DevicePackedExpertBank(gate_up=gate_up, down=down, device=cuda)
+    got = moe_step(torch.from_numpy(hidden).to(cuda), bank, k, logits=torch.from_numpy(logits).to(cuda))
+    assert rel_l2(got.cpu().numpy(), want) <= 2e-5
+
+
+def test_experts_inference_dispatch_with_given_routing_and_empty_experts(cuda):
+    e, d, f, k = 32, 256, 256, 3
+    gate, up, down, _, _ = make_layer(e, d, f, 256, ("Q8_0", "Q8_0", "Q8_0"), 500)
+    rng = np.random.default_rng(1)
+    x = rng.normal(0, 2, (2, 5, d)).astype(np.float32)
+    ids = np.stack([rng.choice(8, k, replace=False) for _ in range(10)]).reshape(2, 5, k)  # experts 8..31 stay empty
+    w = rng.random((2, 5, k)).astype(np.float32)
+
+    def expert_fn(i, rows):
+        return R.expert_ffn(rows, triple(gate.select_outer(i)), triple(up.select_outer(i)), triple(down.select_outer(i)))
+
+    want = R.experts_forward(x.reshape(10, d), w.reshape(10, k), ids.reshape(10, k), e, expert_fn)
+    layer = ExpertsInference(d, f, e, expert_executor=DevicePackedExpertBank(gate, up, down, device=cuda))
+    called = []
+    got = layer.forward(torch.from_numpy(x).to(cuda), torch.from_numpy(w).to(cuda), torch.from_numpy(ids).to(cuda),
+                        on_cpu_submitted=lambda: called.append(1))
+    assert got.shape == (2, 5, d) and called == [1]
+    assert rel_l2(got.reshape(10, d).cpu().numpy(), want) <= 2e-5
+    with pytest.raises(ValueError, match="dimensions"):
+        ExpertsInference(d, f, e + 1, expert_executor=layer.bank)
+
+
+def test_qwen3next_moe_module_and_zero_gate(cuda):
+    e, d, f, fsh, k = 16, 256, 256, 512, 4
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh, ("Q8_0", "Q8_0", "Q6_K"), 700)
+    rng = np.random.default_rng(77)
+    router_w = rng.normal(0, .3, (e, d)).astype(np.float32)
+    hidden = rng.normal(0, 2, (2, 5, d)).astype(np.float32)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    dshared = tuple(upload(w, cuda) for w in shared)
+    for vec in (gate_vec, np.zeros_like(gate_vec)):
+        moe = Qwen3NextMoEInference(bank, k, torch.from_numpy(router_w).to(cuda), dshared, torch.from_numpy(vec).to(cuda))
+        hd = torch.from_numpy(hidden).to(cuda)
+        logits = (hd.reshape(10, d) @ moe.router.W_router).cpu().numpy()
+        assert not synthetic.has_topk_ties(logits, k)
+        want, _, _ = oracle_step(hidden.reshape(10, d), logits, k, gate, up, down, shared, vec)
+        got = moe.forward(hd)
+        assert got.shape == hidden.shape
+        assert rel_l2(got.reshape(10, d).cpu().numpy(), want) <= 2e-5
+    assert moe.forward(hd[:, :0]).shape == (2, 0, d)
+    with pytest.raises(TypeError, match="float32"):
+        moe.forward(hd.half())
+    with pytest.raises(ValueError, match="shape"):
+        moe.forward(hd[0])
+
+
+def test_combine_order_is_ascending_expert_id(cuda):
+    """Three experts whose outputs are 4e20*x, -8e20*x and 6*x-like magnitudes: only the
+    ascending-expert order cancels the large terms first (slot order would lose the small one)."""
+    d = f = 256
+    e = 3
+    # identity-like experts are not expressible in packed form; use the plan + combine alone
+    # through precomputed terms: route weights carry the magnitudes, expert outputs are equal.
+    gate, up, down, _, _ = make_layer(e, d, f, 256, ("Q8_0", "Q8_0", "Q8_0"), 900)
+    # make the three experts identical so that out_e(x) is the same vector v
+    one = gate.select_outer(0).data
+    g = synthetic.packed_weight("Q8_0", (e, f, d), 1); g.data[:] = np.tile(one, e)
+    one = up.select_outer(0).data
+    u = synthetic.packed_weight("Q8_0", (e, f, d), 1); u.data[:] = np.tile(one, e)
+    one = down.select_outer(0).data
+    dn = synthetic.packed_weight("Q8_0", (e, d, f), 1); dn.data[:] = np.tile(one, e)
+    x = synthetic.activations((1, d), 5) * np.float32(4.0)
+    v = R.expert_ffn(x, triple(g.select_outer(0)), triple(u.select_outer(0)), triple(dn.select_outer(0)))
+    ids = np.array([[2, 0, 1]], np.int64)
+    w = np.array([[3.0, 1e8, -1e8]], np.float32)   # slot order: 3, 1e8, -1e8 ; expert order: 1e8, -1e8, 3
+    want = ((np.float32(0) + np.float32(1e8) * v) + np.float32(-1e8) * v) + np.float32(3.0) * v
+    bank = DevicePackedExpertBank(g, u, dn, device=cuda)
+    got = moe_step(torch.from_numpy(x).to(cuda), bank, 3, weights=torch.from_numpy(w).to(cuda),
+                   ids=torch.from_numpy(ids).to(cuda)).cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6 * np.abs(want).max())
+    slot_order = ((np.float32(0) + np.float32(3.0) * v) + np.float32(1e8) * v) + np.float32(-1e8) * v
+    assert rel_l2(slot_order, want) > 0.1  # the wrong order is far away, so the check has teeth
+
+
+# ---- grouped single-token decode (pointer table) ------------------------------------------------
+FORMATS = [("Q8_0", "Q8_0", "Q8_0"), ("Q5_K", "Q4_K", "Q6_K"), ("Q6_K", "Q6_K", "Q6_K")]
+
+
+def handles(formats, cuda, d=256, f=256, count=3, seed=10600):
+    hosts = [tuple(synthetic.packed_weight(fmt, (n, k), seed + 3 * i + j)
+                   for j, (fmt, n, k) in enumerate(zip(formats, (f, f, d), (d, d, f)))) for i in range(count)]
+    dev = [PackedExpertFFNInference(*(upload(w, cuda) for w in h)) for h in hosts]
+    return hosts, dev
+
+
+@pytest.mark.parametrize("formats", FORMATS)
+def test_grouped_decode_matches_oracle(cuda, formats):
+    announce("grouped", formats)
+    hosts, dev = handles(formats, cuda, d=768 if formats[0] != "Q8_0" else 256)
+    d = hosts[0][0].shape[1]
+    x = np.random.default_rng(107).normal(0, 2, (1, d)).astype(np.float32)
+    routes_host = np.array([.7, -.2, .3, 0], np.float32)
+    order = [0, 1, 0, 2]  # the same expert allocation may appear twice
+    selected = [tuple(triple(w) for w in hosts[i]) for i in order]
+    want = R.grouped_decode(x, selected, routes_host)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        xd = torch.from_numpy(x).to(cuda)
+        routes = torch.from_numpy(np.repeat(routes_host, 2)).to(cuda)[::2]  # strided view
+        hs = [dev[i] for i in order]
+        assert supports_grouped_quantized_experts(xd, hs, routes)
+        got = grouped_quantized_experts_forward(xd, hs, routes)
+    stream.synchronize()
+    assert got.shape == (1, d) and got.dtype == torch.float32 and got.data_ptr() != xd.data_ptr()
+    assert rel_l2(got.cpu().numpy(), want) <= 2e-5
+    np.testing.assert_array_equal(xd.cpu().numpy(), x)
+    # slot indirection is bitwise equal to materialised routes
+    slots = (2, 0, 3, 1)
+    a = grouped_quantized_experts_forward(xd, hs, routes.contiguous(), routing_slots=slots)
+    b = grouped_quantized_experts_forward(xd, hs, routes.contiguous()[list(slots)].contiguous())
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("case,reason", [
+    ("batch", "contiguous"), ("noncontiguous", "contiguous"), ("dtype", "FP32"),
+    ("routes_shape", "routing_weights"), ("routes_dtype", "routing_weights"),
+    ("empty", "nonempty"), ("handle", "handles"), ("mixed", "per-projection"), ("shapes", "shapes"),
+    ("block", "block_k"), ("slots", "routing_slots")])
+def test_grouped_decode_rejections(cuda, case, reason):
+    hosts, dev = handles(FORMATS[0], cuda, count=1)
+    x = torch.zeros((1, 256), device=cuda)
+    routes = torch.ones(1, device=cuda)
+    kwargs = {}
+    if case == "batch":
+        x = torch.zeros((2, 256), device=cuda)
+    elif case == "noncontiguous":
+        x = torch.zeros((1, 512), device=cuda)[:, ::2]
+    elif case == "dtype":
+        x = x.half()
+    elif case == "routes_shape":
+        routes = routes.reshape(1, 1)
+    elif case == "routes_dtype":
+        routes = routes.double()
+    elif case == "empty":
+        dev = []
+    elif case == "handle":
+        dev = [object()]
+    elif case == "mixed":
+        dev = dev + handles(FORMATS[1], cuda, count=1)[1]
+        routes = torch.ones(2, device=cuda)
+    elif case == "shapes":
+        x = torch.zeros((1, 512), device=cuda)
+    elif case == "block":
+        kwargs["block_k"] = 128
+    elif case == "slots":
+        kwargs["routing_slots"] = (1,)
+    assert not supports_grouped_quantized_experts(x, dev, routes, **kwargs)
+    with pytest.raises(ValueError, match=reason):
+        grouped_quantized_experts_forward(x, dev, routes, **kwargs)
+
+
+def test_grouped_ordered_reduce_is_sequential_not_tree(cuda):
+    # equal experts, routes 1e8, 1, -1e8, 3: sequential fp32 adds give 3*v-ish cancellation
+    hosts, dev = handles(FORMATS[0], cuda, count=1)
+    x = np.random.default_rng(108).normal(0, 2, (1, 256)).astype(np.float32)
+    routes = np.array([1e8, 1, -1e8, 3], np.float32)
+    sel = [tuple(triple(w) for w in hosts[0])] * 4
+    want = R.grouped_decode(x, sel, routes)
+    got = grouped_quantized_experts_forward(torch.from_numpy(x).to(cuda), dev * 4, torch.from_numpy(routes).to(cuda))
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-6 * np.abs(want).max())
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K"])
+@pytest.mark.parametrize("tokens", [1, 4, 16])
+def test_decode_config_512_experts_top10(cuda, fmt, tokens):
+    """Benchmark decode configuration at full shape: D=2048, 512 experts, top-10, F=512,
+    shared F=2048.  Checked through sampled tokens against the oracle (the oracle decodes
+    only the experts those tokens selected)."""
+    announce("moe decode full", fmt, tokens)
+    e, d, f, fsh, k = 512, 2048, 512, 2048, 10
+    gate, up, down, shared, gate_vec, bank, dshared = full_layer(fmt, cuda)
+    hidden = synthetic.activations((tokens, d), 7, "bf16")
+    logits = synthetic.router_logits(tokens, e, 9)
+    assert not synthetic.has_topk_ties(logits, k)
+    out, w, ids = moe_step(torch.from_numpy(hidden).to(cuda), bank, k, logits=torch.from_numpy(logits).to(cuda),
+                           shared=dshared, shared_gate=torch.from_numpy(gate_vec).to(cuda), return_routing=True)
+    sample = sorted(set([0, tokens - 1]))
+    want, want_w, want_ids = oracle_step(hidden[sample], logits[sample], k, gate, up, down, shared, gate_vec)
+    np.testing.assert_array_equal(ids.cpu().numpy()[sample], want_ids)
+    np.testing.assert_allclose(w.cpu().numpy()[sample], want_w, rtol=2e-6, atol=2e-7)
+    assert rel_l2(out.cpu().numpy()[sample], want) <= 2e-5 <= REL_L2
+
+
+def test_prefill_config_512_tokens_zipf(cuda):
+    """Benchmark prefill configuration: T=512, Zipf(1.1) routing, Q8_0.  Size-independent
+    checks: every token's output equals the same token run alone (dispatch/compaction is
+    permutation-invariant), plus sampled tokens against the oracle."""
+    announce("moe prefill T=512")
+    e, d, f, fsh, k, t = 512, 2048, 512, 2048, 10, 512
+    gate, up, down, shared, gate_vec, bank, dshared = full_layer("Q8_0", cuda)
+    hidden = synthetic.activations((t, d), 7, "bf16")
+    logits = synthetic.router_logits(t, e, 9, zipf=1.1)
+    assert not synthetic.has_topk_ties(logits, k)
+    hd, ld, gd = torch.from_numpy(hidden).to(cuda), torch.from_numpy(logits).to(cuda), torch.from_numpy(gate_vec).to(cuda)
+    out, w, ids = moe_step(hd, bank, k, logits=ld, shared=dshared, shared_gate=gd, return_routing=True)
+    counts = np.bincount(ids.cpu().numpy().ravel(), minlength=e)
+    assert counts.max() > 5 * counts.mean()  # the routing really is skewed
+    picks = [0, 17, 255, 511]
+    for i in picks:
+        alone = moe_step(hd[i:i + 1].contiguous(), bank, k, logits=ld[i:i + 1].contiguous(), shared=dshared, shared_gate=gd)
+        assert rel_l2(out[i:i + 1].cpu().numpy(), alone.cpu().numpy()) <= 1e-5
+    want, _, want_ids = oracle_step(hidden[picks[:2]], logits[picks[:2]], k, gate, up, down, shared, gate_vec)
+    np.testing.assert_array_equal(ids.cpu().numpy()[picks[:2]], want_ids)
+    assert rel_l2(out.cpu().numpy()[picks[:2]], want) <= 2e-5

@@ -1,0 +1,141 @@
+"""Host-side logic that needs no GPU: the packed container, the ABI surface of the built
+library, and argument validation that returns before any kernel would be launched."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from mylocal_llm_amd import _lib, synthetic
+from mylocal_llm_amd.quantized_weight import BLOCK_FORMATS, PackedGGUFWeight
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_block_format_table():
+    assert BLOCK_FORMATS["Q8_0"] == (32, 34)
+    assert BLOCK_FORMATS["Q5_K"] == (256, 176)
+    assert BLOCK_FORMATS["Q6_K"] == (256, 210)
+    assert BLOCK_FORMATS["Q4_K"] == (256, 144)
+    assert BLOCK_FORMATS["Q4_0"] == (32, 18)
+
+
+@pytest.mark.parametrize("fmt", list(BLOCK_FORMATS))
+def test_length_alignment_and_type_errors(fmt):
+    elems, nbytes = BLOCK_FORMATS[fmt]
+    good = np.zeros(2 * nbytes, np.uint8)
+    PackedGGUFWeight(good, (1, 2 * elems), fmt)
+    with pytest.raises(ValueError, match="expected"):
+        PackedGGUFWeight(good[:-1], (1, 2 * elems), fmt)
+    if elems > 1:
+        with pytest.raises(ValueError, match="innermost"):
+            PackedGGUFWeight(good, (1, 2 * elems - 1), fmt)
+    with pytest.raises(ValueError, match="Unsupported"):
+        PackedGGUFWeight(good, (1, 2 * elems), "Q9_Z")
+    with pytest.raises(ValueError, match="positive"):
+        PackedGGUFWeight(good, (0, 2 * elems), fmt)
+    with pytest.raises(ValueError, match="contiguous"):
+        PackedGGUFWeight(np.zeros(4 * nbytes, np.uint8)[::2], (1, 2 * elems), fmt)
+
+
+def test_select_outer_and_rows_are_zero_copy():
+    original = synthetic.packed_weight("Q5_K", (3, 4, 512), 49)
+    sample = original.select_outer(1)
+    assert sample.shape == (4, 512) and sample.nbytes == 4 * 2 * 176
+    assert np.shares_memory(sample.data, original.data)
+    np.testing.assert_array_equal(sample.data, original.data[sample.nbytes:2 * sample.nbytes])
+    rows = sample.select_rows(1, 3)
+    assert rows.shape == (2, 512) and np.shares_memory(rows.data, original.data)
+    with pytest.raises(IndexError):
+        original.select_outer(3)
+    with pytest.raises(ValueError):
+        sample.select_outer(0).select_outer(0)
+
+
+def test_mmap_payload_stays_the_owner(tmp_path):
+    w = synthetic.packed_weight("Q6_K", (12, 512), 5)
+    path = tmp_path / "q6.bin"
+    path.write_bytes(w.data.tobytes())
+    mapped = np.memmap(path, dtype=np.uint8, mode="r")
+    view = PackedGGUFWeight(mapped, (3, 4, 512), "Q6_K").select_outer(2)
+    assert np.shares_memory(view.data, mapped)
+    np.testing.assert_array_equal(view.data, w.data[2 * view.nbytes:])
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qmoe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qmoe_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert set(names) == set(_lib.EXPORTS)
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert lib.qmoe_abi_version() == 1
+
+
+def test_format_info_matches_table():
+    lib = _lib.load()
+    e, b = ctypes.c_int(), ctypes.c_int()
+    for fmt, (elems, nbytes) in BLOCK_FORMATS.items():
+        assert lib.qmoe_format_info(_lib.FORMAT_ID[fmt], ctypes.byref(e), ctypes.byref(b)) == 0
+        assert (e.value, b.value) == (elems, nbytes)
+    assert lib.qmoe_format_info(77, ctypes.byref(e), ctypes.byref(b)) == 1
+    assert b"unknown" in lib.qmoe_last_error()
+
+
+def test_invalid_arguments_return_codes_before_any_launch():
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    fake = ctypes.c_void_p(4096)  # never dereferenced: validation fails first
+    assert lib.qmoe_linear(null, 0, 4, 32, fake, 0, 1, fake, 0, null) == 1
+    assert lib.qmoe_linear(fake, 0, 4, 33, fake, 0, 1, fake, 0, null) == 1      # K not a block multiple
+    assert b"multiple" in lib.qmoe_last_error()
+    assert lib.qmoe_linear(fake, 0, 4, 32, fake, 0, 0, fake, 0, null) == 1      # no tokens
+    assert lib.qmoe_linear(fake, 3, 4, 256, fake, 0, 1, fake, 0, null) == 2     # Q3_K: recognised, no kernel
+    assert lib.qmoe_linear(fake, 42, 4, 256, fake, 0, 1, fake, 0, null) == 1    # unknown format
+    assert lib.qmoe_linear(fake, 0, 4, 32, fake, 9, 1, fake, 0, null) == 1      # unknown dtype
+    assert lib.qmoe_dequantize(fake, 5, 2, 100, fake, null) == 1
+    assert lib.qmoe_swiglu(fake, 0, null, 0, 4, 32, fake, 0, 1, fake, 0, null) == 1
+    assert lib.qmoe_expert(fake, 0, fake, 0, fake, 0, 32, 32, fake, 0, 1, fake, 0, null, null) == 4
+    assert lib.qmoe_router_topk(fake, 1, 5000, 2, 1e-6, 1, fake, fake, null) == 2
+    assert lib.qmoe_router_topk(fake, 1, 16, 33, 1e-6, 1, fake, fake, null) == 2
+    assert lib.qmoe_router_topk(fake, 1, 16, 3, 1e-50, 1, fake, fake, null) == 1
+    assert lib.qmoe_grouped_decode(fake, fake, 0, 0, 0, 0, 32, 32, fake, 1, null, fake, fake, null) == 1
+    assert lib.qmoe_moe_forward(None, null, 0, null) == 1
+
+
+def test_moe_workspace_size_is_monotone_and_aligned():
+    lib = _lib.load()
+    a = lib.qmoe_moe_workspace_bytes(1, 10, 512, 2048, 512, 2048)
+    b = lib.qmoe_moe_workspace_bytes(16, 10, 512, 2048, 512, 2048)
+    assert 0 < a < b and a % 256 == 0 and b % 256 == 0
+    assert lib.qmoe_moe_workspace_bytes(1, 0, 512, 2048, 512, 0) == 0
+
+
+def test_host_weights_have_no_compute_path():
+    torch = pytest.importorskip("torch")
+    from mylocal_llm_amd.quantized_linear import quantized_linear, quantized_swiglu, packed_to_device
+    w = synthetic.packed_weight("Q4_K", (2, 256), 1)
+    with pytest.raises(TypeError, match="NumPy"):
+        quantized_linear(np.zeros((2, 256), np.float32), w)
+    with pytest.raises(TypeError, match="NumPy"):
+        quantized_linear([[0] * 256], w)
+    with pytest.raises(TypeError):
+        quantized_swiglu(np.zeros((2, 256), np.float32), w, w)
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="HIP device"):
+            packed_to_device(w)
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "mylocal_llm_amd")
+    for base, _, files in os.walk(pkg):
+        for name in files:
+            if name.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(base, name)).read()
+                assert "oracle" not in text.replace("no oracle", ""), os.path.join(base, name)
