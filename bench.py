@@ -1,0 +1,269 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed-weight decode path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): Llama-3-8B-shaped Q8_0 projections at M=1,
+all seven projections of a layer, 32 layers streamed back-to-back.  One "step" is one
+token's pass over the 32 layers (224 packed matrices, 7 415 529 472 weight bytes, every one
+read once).  `value` is weight-bytes-effective GB/s of the whole step with all inputs
+resident in HBM; tokens/s of the same stream is in `config`.
+
+The JSON line also carries
+  roofline      achieved HBM GB/s of the dominant kernel (algorithmic bytes per launch over
+                its average launch duration, from HIP events on the launch stream)
+  cpu_baseline  the NumPy restatement of the reference's packed CPU path (dequantise on every
+                call, fp32 matmul) timed on this box's host cores on a bounded sample
+  extras        other configurations (formats, token counts, MoE decode) measured the same way
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+# (name, N, K) of the seven projections of one Llama-3-8B layer
+PROJECTIONS = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+               ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
+BLOCKS = {"Q8_0": (32, 34), "Q5_K": (256, 176), "Q6_K": (256, 210), "BF16": (1, 2)}
+
+
+def weight_bytes(fmt, n, k):
+    e, b = BLOCKS[fmt]
+    return n * k // e * b
+
+
+def device_blocks(torch, fmt, n, k, gen, device):
+    """Synthetic packed matrix [n, k] generated on the device with the distribution the
+    workload names (see mylocal_llm_amd/synthetic.py for the host twin)."""
+    e, b = BLOCKS[fmt]
+    nb = n * k // e
+    blk = torch.empty((nb, b), dtype=torch.uint8, device=device)
+
+    def scale(count):
+        return (torch.randn(count, device=device, generator=gen) * 1e-4 + 5e-4).abs().to(torch.float16).view(torch.uint8).reshape(count, 2)
+
+    if fmt == "Q8_0":
+        q = (torch.randn((nb, 32), device=device, generator=gen) * 40).round().clamp(-127, 127).to(torch.int8)
+        blk[:, 0:2] = scale(nb)
+        blk[:, 2:] = q.view(torch.uint8)
+    elif fmt == "Q6_K":
+        blk[:, 0:192] = torch.randint(0, 256, (nb, 192), device=device, generator=gen, dtype=torch.uint8)
+        blk[:, 192:208] = torch.randint(-64, 64, (nb, 16), device=device, generator=gen, dtype=torch.int8).view(torch.uint8)
+        blk[:, 208:210] = scale(nb)
+    elif fmt == "Q5_K":
+        blk[:, 0:2] = scale(nb)
+        blk[:, 2:4] = scale(nb)
+        # any 12 bytes are a valid field of eight 6-bit (scale, min) pairs, uniform over 0..63
+        blk[:, 4:] = torch.randint(0, 256, (nb, b - 4), device=device, generator=gen, dtype=torch.uint8)
+    elif fmt == "BF16":
+        v = (torch.randn(nb, device=device, generator=gen) * 0.02).to(torch.bfloat16)
+        blk[:] = v.view(torch.uint8).reshape(nb, 2)
+    else:
+        raise ValueError(fmt)
+    return blk.reshape(-1)
+
+
+class LayerStream:
+    """`layers` x 7 packed projections resident in HBM plus activation / output buffers."""
+
+    def __init__(self, torch, lib, fmt, layers, tokens, device, seed=106):
+        from mylocal_llm_amd import _lib
+        self.torch, self.lib, self.fmt, self.layers, self.tokens = torch, lib, fmt, layers, tokens
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed)
+        self.weights = [[device_blocks(torch, fmt, n, k, gen, device) for _, n, k in PROJECTIONS] for _ in range(layers)]
+        xgen = torch.Generator(device=device)
+        xgen.manual_seed(103)
+        # one activation buffer per data-flow group: (q, k, v) share the layer input, o reads the
+        # attention output, (gate, up) the post-attention state, down the SwiGLU activation
+        self.x = {name: torch.randn((tokens, k), device=device, generator=xgen)
+                  for name, k in (("qkv", 4096), ("o", 4096), ("gateup", 4096), ("down", 14336))}
+        group = {"q": "qkv", "k": "qkv", "v": "qkv", "o": "o", "gate": "gateup", "up": "gateup", "down": "down"}
+        self.y = [torch.empty((tokens, n), device=device) for _, n, _ in PROJECTIONS]
+        self.bytes_per_layer = sum(weight_bytes(fmt, n, k) for _, n, k in PROJECTIONS)
+        fid = _lib.FORMAT_ID[fmt]
+        self.batches = []
+        for layer in range(layers):
+            arr = (_lib.LinearProblem * len(PROJECTIONS))()
+            for i, (name, n, k) in enumerate(PROJECTIONS):
+                p = arr[i]
+                p.w, p.x, p.y = self.weights[layer][i].data_ptr(), self.x[group[name]].data_ptr(), self.y[i].data_ptr()
+                p.fmt, p.n, p.k, p.tokens, p.x_dtype, p.y_dtype = fid, n, k, tokens, 0, 0
+            self.batches.append(arr)
+        self.launches_per_step = layers  # one batched launch sequence per layer
+
+    def step(self, stream):
+        lib = self.lib
+        for arr in self.batches:
+            rc = lib.qmoe_linear_batch(arr, len(PROJECTIONS), stream)
+            if rc:
+                raise RuntimeError(lib.qmoe_last_error().decode())
+
+
+def time_steps(torch, fn, steps, warmup):
+    """(wall seconds, event milliseconds) for `steps` calls of fn after `warmup` untimed ones."""
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(warmup):
+        fn(stream)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn(stream)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, start.elapsed_time(stop)
+
+
+def cpu_baseline(budget_s=12.0):
+    """NumPy restatement of the reference's packed CPU path on a bounded sample of the
+    headline workload: the k and q projections of one layer (1024x4096 and 4096x4096 Q8_0,
+    M=1), dequantised on every call as the reference's default host branch does."""
+    import numpy as np
+    from mylocal_llm_amd import synthetic
+    from oracle import reference_np as R
+    sample = [(1024, 4096), (4096, 4096)]
+    ws = [synthetic.packed_weight("Q8_0", s, 106 + i) for i, s in enumerate(sample)]
+    x = synthetic.activations((1, 4096), 103)
+    nbytes = sum(w.nbytes for w in ws)
+    R.linear(x, ws[0].data, ws[0].shape, "Q8_0")  # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        for w in ws:
+            R.linear(x, w.data, w.shape, "Q8_0")
+        reps += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed > budget_s:
+            break
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    return {"value": round(nbytes * reps / elapsed / 1e9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "sample": f"Q8_0 M=1 k-proj 1024x4096 + q-proj 4096x4096 ({nbytes} weight bytes), {reps} repetitions in "
+                      f"{elapsed:.1f}s, NumPy dequantise-every-call + fp32 matmul (oracle/reference_np.linear)",
+            "numpy": np.__version__, "host_cpus": os.cpu_count()}
+
+
+def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup):
+    """512-expert top-10 MoE decode step (D=2048, F=512, shared F=2048) over rotating banks."""
+    from mylocal_llm_amd import _lib
+    from mylocal_llm_amd.moe import DevicePackedExpertBank, moe_step
+    from mylocal_llm_amd.quantized_linear import DevicePackedGGUFWeight
+    e, d, f, fsh, k = 512, 2048, 512, 2048, 10
+    gen = torch.Generator(device=device)
+    gen.manual_seed(7)
+    n_banks = 4  # distinct layers' banks, so that a step never re-reads recently touched bytes
+    banks, shareds = [], []
+    for _ in range(n_banks):
+        g = device_blocks(torch, fmt, e * f, d, gen, device)
+        u = device_blocks(torch, fmt, e * f, d, gen, device)
+        dn = device_blocks(torch, fmt, e * d, f, gen, device)
+        banks.append(DevicePackedExpertBank((g, (e, f, d), fmt), (u, (e, f, d), fmt), (dn, (e, d, f), fmt)))
+        shareds.append(tuple(DevicePackedGGUFWeight(device_blocks(torch, fmt, n, kk, gen, device), (n, kk), fmt)
+                             for n, kk in ((fsh, d), (fsh, d), (d, fsh))))
+    hidden = torch.randn((tokens, d), device=device, generator=gen).to(torch.bfloat16)
+    logits = torch.randn((n_banks, tokens, e), device=device, generator=gen)
+    gate_vec = torch.randn(d, device=device, generator=gen) * 0.02
+    state = {"i": 0}
+
+    def fn(_stream):
+        i = state["i"] % n_banks
+        state["i"] += 1
+        moe_step(hidden, banks[i], k, logits=logits[i], shared=shareds[i], shared_gate=gate_vec)
+
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    # algorithmic bytes: distinct selected experts (averaged over the banks' logits) + shared expert
+    ids = torch.topk(logits, k, dim=-1).indices
+    distinct = sum(len(torch.unique(ids[i])) for i in range(n_banks)) / n_banks
+    eb = 3 * weight_bytes(fmt, f, d)
+    sb = 3 * weight_bytes(fmt, fsh, d)
+    nbytes = distinct * eb + sb
+    per_step = ms / steps * 1e-3
+    return {"workload": f"moe_decode_{fmt}_T{tokens}", "ms_per_step": round(ms / steps, 4),
+            "weight_bytes": int(nbytes), "distinct_experts": distinct,
+            "GBps": round(nbytes / per_step / 1e9, 1), "frac_hbm_peak": round(nbytes / per_step / 1e9 / HBM_PEAK_GBS, 4),
+            "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(no collectives or sharding in this path)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from mylocal_llm_amd import _lib
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.load()
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+
+    stream = LayerStream(torch, lib, "Q8_0", args.layers, 1, device)
+    wall, ms = time_steps(torch, stream.step, args.steps, args.warmup)
+    step_s = wall / args.steps
+    total_bytes = stream.bytes_per_layer * args.layers
+    value = total_bytes / step_s / 1e9
+    launches = args.steps * stream.launches_per_step
+    launch_ms = ms / launches
+    achieved = stream.bytes_per_layer / (launch_ms * 1e-3) / 1e9
+    result = {
+        "metric": "effective weight GB/s (Q8_0 8B projections, M=1, 32 layers streamed)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"configs[1]: Llama-3-8B-shaped Q8_0 projections, M=1, {args.layers} layers x 7 "
+                               "projections streamed back-to-back, one batched launch sequence per layer",
+                   "weight_bytes_per_step": total_bytes, "tokens_per_s": round(1.0 / step_s, 1),
+                   "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4), "activations": "fp32 N(0,1)"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "linear (Q8_0, M=1), one layer = 7 projections per launch sequence",
+                     "bytes_per_launch": stream.bytes_per_layer, "avg_launch_us": round(launch_ms * 1e3, 3)},
+    }
+    del stream
+    torch.cuda.empty_cache()
+    if not args.no_extras:
+        extras = []
+        for fmt, tokens in (("Q6_K", 1), ("Q5_K", 1), ("BF16", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16)):
+            s = LayerStream(torch, lib, fmt, 8, tokens, device)
+            w, m = time_steps(torch, s.step, max(3, args.steps // 4), 2)
+            n = max(3, args.steps // 4)
+            per_layer = m / n / 8 * 1e-3
+            extras.append({"workload": f"8B projections {fmt} M={tokens} (8 layers)",
+                           "GBps": round(s.bytes_per_layer / per_layer / 1e9, 1),
+                           "frac_hbm_peak": round(s.bytes_per_layer / per_layer / 1e9 / HBM_PEAK_GBS, 4),
+                           "us_per_layer": round(per_layer * 1e6, 2),
+                           "tokens_per_s_32_layers": round(tokens / (per_layer * 32), 1)})
+            del s
+            torch.cuda.empty_cache()
+        for fmt, tokens in (("Q8_0", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q6_K", 1)):
+            extras.append(moe_decode_extra(torch, lib, device, fmt, tokens, max(8, args.steps), 3))
+            torch.cuda.empty_cache()
+        result["extras"] = extras
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

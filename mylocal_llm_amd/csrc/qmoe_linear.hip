@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include "qmoe_rowdot.hpp"
+#include "qmoe_stream.hpp"
 
 namespace qmoe {
 
@@ -130,6 +131,12 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
     if ((rc = validate_dtype("qmoe_linear", "input", xdt)) || (rc = validate_dtype("qmoe_linear", "output", ydt))) return rc;
     if ((uintptr_t)x % dtype_size(xdt) || (uintptr_t)y % dtype_size(ydt))
         return fail(QMOE_EINVAL, "qmoe_linear: activation/output pointer not aligned to its element type");
+    if (tokens == 1 && stream_supported(fmt, w, n, k, x, xdt)) {
+        StreamArgs args{};
+        args.count = 1;
+        args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, fmt, xdt, ydt, 0, 0};
+        return stream_launch(args, s);
+    }
     const bool fast = rows_fast(fmt, w, row_bytes(fmt, k), k) && x_fast(x, xdt, k);
     if (xdt == QMOE_DT_F32) launch_linear_mt<QMOE_DT_F32>(w, fmt, n, k, fast, x, tokens, y, ydt, s);
     else if (xdt == QMOE_DT_F16) launch_linear_mt<QMOE_DT_F16>(w, fmt, n, k, fast, x, tokens, y, ydt, s);
@@ -186,6 +193,12 @@ int swiglu_impl(const void* gate, int gf, const void* up, int uf, int f, int k, 
     if ((rc = validate_dtype("qmoe_swiglu", "input", xdt)) || (rc = validate_dtype("qmoe_swiglu", "output", hdt))) return rc;
     if ((uintptr_t)x % dtype_size(xdt) || (uintptr_t)h % dtype_size(hdt))
         return fail(QMOE_EINVAL, "qmoe_swiglu: activation/output pointer not aligned to its element type");
+    if (tokens == 1 && gf == uf && stream_supported(gf, gate, f, k, x, xdt) && stream_supported(uf, up, f, k, x, xdt)) {
+        StreamArgs args{};
+        args.count = 1;
+        args.p[0] = StreamProblem{(const uint8_t*)gate, (const uint8_t*)up, x, h, f, k, gf, uf, xdt, hdt, 0, 0};
+        return stream_launch(args, s);
+    }
     const bool xf = x_fast(x, xdt, k);
     const bool gfast = xf && rows_fast(gf, gate, row_bytes(gf, k), k);
     const bool ufast = xf && rows_fast(uf, up, row_bytes(uf, k), k);
@@ -241,10 +254,31 @@ int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stre
         if (!p.x || !p.y || p.tokens < 1 || !dtype_size(p.x_dtype) || !dtype_size(p.y_dtype))
             return fail(QMOE_EINVAL, "qmoe_linear_batch: problem %d has a null pointer, no tokens or a bad element type", i);
     }
+    // Single-token problems the streaming kernel covers share launches (up to
+    // STREAM_MAX_PROBLEMS each); anything else goes through the general kernels in order.
+    StreamArgs args{};
     for (int i = 0; i < count; ++i) {
         const qmoe_linear_problem& p = problems[i];
-        int rc = linear_impl(p.w, p.fmt, p.n, p.k, p.x, p.x_dtype, p.tokens, p.y, p.y_dtype, (hipStream_t)stream);
-        if (rc) return rc;
+        const bool ok = p.tokens == 1 && (uintptr_t)p.x % dtype_size(p.x_dtype) == 0 &&
+                        (uintptr_t)p.y % dtype_size(p.y_dtype) == 0 && stream_supported(p.fmt, p.w, p.n, p.k, p.x, p.x_dtype);
+        if (ok && args.count && args.p[0].fmt != p.fmt) {  // one packed format per launch
+            int rc = stream_launch(args, (hipStream_t)stream);
+            if (rc) return rc;
+            args.count = 0;
+        }
+        if (ok) {
+            args.p[args.count++] = StreamProblem{(const uint8_t*)p.w, nullptr, p.x, p.y, p.n, p.k, p.fmt, p.fmt,
+                                                 p.x_dtype, p.y_dtype, 0, 0};
+        }
+        if (args.count == STREAM_MAX_PROBLEMS || (!ok && args.count) || (i == count - 1 && args.count)) {
+            int rc = stream_launch(args, (hipStream_t)stream);
+            if (rc) return rc;
+            args.count = 0;
+        }
+        if (!ok) {
+            int rc = linear_impl(p.w, p.fmt, p.n, p.k, p.x, p.x_dtype, p.tokens, p.y, p.y_dtype, (hipStream_t)stream);
+            if (rc) return rc;
+        }
     }
     return QMOE_OK;
 }

@@ -1,0 +1,260 @@
+// Single-token weight-streaming engine: one pass over packed rows at HBM speed.
+//
+// Every format is cut into 64-element lane units.  A lane keeps the 64 activation values
+// of its unit position in registers for the whole problem, loads its unit of each row
+// straight from global memory with the widest loads the block layout allows, decodes in
+// registers and accumulates in fp32; one row (or one gate/up row pair) costs one DPP
+// reduction across the lanes that share it.  Rows are never staged in LDS: consecutive
+// lanes read consecutive units, so a wave's loads cover one contiguous stretch of the row.
+//
+//   Q8_0  unit = 2 blocks            68 B  (4 x 16 B + 4 B)
+//   Q6_K  unit = quarter block       48 B + 8 B scales + 2 B d   (16-lane runs of 4 quarters)
+//   Q5_K  unit = quarter block       40 B + 16 B header          (8-lane runs of 8 groups)
+//   BF16  unit = 64 elements        128 B
+#pragma once
+#include "qmoe_common.hpp"
+#include "qmoe_formats.hpp"
+
+namespace qmoe {
+
+// ---- DPP reductions -----------------------------------------------------------------------
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_add(float v) {
+    int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false);
+    return v + __int_as_float(r);
+}
+// Sum over groups of LR consecutive lanes (LR = 8, 16, 32 or 64).  The total of a group is
+// valid in its last lane.
+template <int LR>
+__device__ __forceinline__ float group_sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror: lanes of an 8-group now agree
+    if (LR >= 16) v = dpp_add<0x140>(v);        // row_mirror: 16 lanes
+    if (LR >= 32) v = dpp_add<0x142, 0xa>(v);   // row_bcast15: lanes 16..31 / 48..63 gain the row before
+    if (LR >= 64) v = dpp_add<0x143, 0xc>(v);   // row_bcast31: lanes 32..63 gain lanes 0..31
+    return v;
+}
+
+struct __attribute__((packed, aligned(2))) u32x4_a2 { uint32_t v[4]; };
+struct __attribute__((packed, aligned(2))) u32x2_a2 { uint32_t v[2]; };
+struct __attribute__((packed, aligned(2))) u32_a2 { uint32_t v; };
+
+__device__ __forceinline__ float ubyte_f(uint32_t w, int i) {
+    // v_cvt_f32_ubyte{0..3}
+    return (float)((w >> (8 * i)) & 0xFFu);
+}
+
+// Activation loader: 4 consecutive elements of any supported type as fp32.
+__device__ __forceinline__ float4 load_x4(const void* x, int xdt, int i) {
+    if (xdt == QMOE_DT_F32) return Elem<QMOE_DT_F32>::load4(x, i);
+    if (xdt == QMOE_DT_F16) return Elem<QMOE_DT_F16>::load4(x, i);
+    return Elem<QMOE_DT_BF16>::load4(x, i);
+}
+
+template <int FMT> struct Unit64;
+
+// ---- Q8_0 -----------------------------------------------------------------------------------
+template <> struct Unit64<QMOE_FMT_Q8_0> {
+    static constexpr int RAW = 17, AUX = 1;
+    static constexpr int ROW_ALIGN = 4;
+    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float*) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float4 v = load_x4(x, xdt, u * 64 + 4 * i);
+            xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+        }
+    }
+    __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
+        const uint8_t* p = row + (size_t)u * 68;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u32x4_a4 v = *(const u32x4_a4*)(p + 16 * i);
+            r[4 * i] = v.v[0]; r[4 * i + 1] = v.v[1]; r[4 * i + 2] = v.v[2]; r[4 * i + 3] = v.v[3];
+        }
+        r[16] = *(const uint32_t*)(p + 64);
+    }
+    __device__ __forceinline__ static float dot(const uint32_t* r, const float* xr, const float*) {
+        const float d0 = half_bits_to_float(r[0] & 0xFFFFu), d1 = half_bits_to_float(r[8] >> 16);
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int b0 = 2 + i, b1 = 36 + i;
+            s0 += sbyte(r[b0 >> 2], b0 & 3) * xr[i];
+            s1 += sbyte(r[b1 >> 2], b1 & 3) * xr[32 + i];
+        }
+        return d0 * s0 + d1 * s1;
+    }
+};
+
+// ---- Q6_K -----------------------------------------------------------------------------------
+// unit u: block u/4, half h = (u/2)%2, column group c = u%2; element (quarter q, j) of the
+// unit is block element 128h + 32q + 16c + j.
+template <> struct Unit64<QMOE_FMT_Q6_K> {
+    static constexpr int RAW = 15, AUX = 4;
+    static constexpr int ROW_ALIGN = 2;
+    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float* aux) {
+        const int base = (u >> 2) * 256 + ((u >> 1) & 1) * 128 + (u & 1) * 16;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float4 v = load_x4(x, xdt, base + 32 * q + 4 * i);
+                xr[16 * q + 4 * i] = v.x; xr[16 * q + 4 * i + 1] = v.y; xr[16 * q + 4 * i + 2] = v.z; xr[16 * q + 4 * i + 3] = v.w;
+                s += (v.x + v.y) + (v.z + v.w);
+            }
+            aux[q] = 32.0f * s;
+        }
+    }
+    __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
+        const uint8_t* b = row + (size_t)(u >> 2) * 210;
+        const int h = (u >> 1) & 1, c = u & 1;
+        u32x4_a2 la = *(const u32x4_a2*)(b + 64 * h + 16 * c);
+        u32x4_a2 lb = *(const u32x4_a2*)(b + 64 * h + 32 + 16 * c);
+        u32x4_a2 hq = *(const u32x4_a2*)(b + 128 + 32 * h + 16 * c);
+        u32x2_a2 sc = *(const u32x2_a2*)(b + 192 + 8 * h);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { r[i] = la.v[i]; r[4 + i] = lb.v[i]; r[8 + i] = hq.v[i]; }
+        // the four sub-block scales of this unit are bytes c, c+2, c+4, c+6 of the half's eight
+        const uint32_t s0 = sc.v[0] >> (8 * c), s1 = sc.v[1] >> (8 * c);
+        r[12] = (s0 & 0xFFu) | ((s0 >> 8) & 0xFF00u);         // scales of quarters 0, 1
+        r[13] = (s1 & 0xFFu) | ((s1 >> 8) & 0xFF00u);         // scales of quarters 2, 3
+        r[14] = ld_u16(b + 208);
+    }
+    __device__ __forceinline__ static float dot(const uint32_t* r, const float* xr, const float* aux) {
+        const float d = half_bits_to_float(r[14]);
+        float total = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float acc = 0.f;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const uint32_t src = (q & 1) ? r[4 + m] : r[m];
+                const uint32_t lo = (q & 2) ? ((src >> 4) & 0x0F0F0F0Fu) : (src & 0x0F0F0F0Fu);
+                const uint32_t hi = (r[8 + m] >> (2 * q)) & 0x03030303u;
+                const uint32_t code = lo | (hi << 4);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc += ubyte_f(code, j) * xr[16 * q + 4 * m + j];
+            }
+            const float scale = d * sbyte(r[12 + (q >> 1)], q & 1);
+            total += scale * (acc - aux[q]);
+        }
+        return total;
+    }
+};
+
+// ---- Q5_K -----------------------------------------------------------------------------------
+// unit u: block u/4, byte column c = u%4; element (group g, j) of the unit is block element
+// 32g + 8c + j.
+template <> struct Unit64<QMOE_FMT_Q5_K> {
+    static constexpr int RAW = 14, AUX = 8;
+    static constexpr int ROW_ALIGN = 16;
+    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float* aux) {
+        const int base = (u >> 2) * 256 + (u & 3) * 8;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            float4 a = load_x4(x, xdt, base + 32 * g), b = load_x4(x, xdt, base + 32 * g + 4);
+            xr[8 * g] = a.x; xr[8 * g + 1] = a.y; xr[8 * g + 2] = a.z; xr[8 * g + 3] = a.w;
+            xr[8 * g + 4] = b.x; xr[8 * g + 5] = b.y; xr[8 * g + 6] = b.z; xr[8 * g + 7] = b.w;
+            aux[g] = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+        }
+    }
+    __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
+        const uint8_t* b = row + (size_t)(u >> 2) * 176;
+        const int c = u & 3;
+        const uint4 hdr = *(const uint4*)b;
+        r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
+        const uint2 qh = *(const uint2*)(b + 16 + 8 * c);
+        r[4] = qh.x; r[5] = qh.y;
+#pragma unroll
+        for (int g2 = 0; g2 < 4; ++g2) {
+            const uint2 qs = *(const uint2*)(b + 48 + 32 * g2 + 8 * c);
+            r[6 + 2 * g2] = qs.x; r[7 + 2 * g2] = qs.y;
+        }
+    }
+    __device__ __forceinline__ static float dot(const uint32_t* r, const float* xr, const float* aux) {
+        const float d = half_bits_to_float(r[0] & 0xFFFFu), dmin = half_bits_to_float(r[0] >> 16);
+        // 6-bit scales / minima of the eight groups, four per dword
+        const uint32_t sc_lo = r[1] & 0x3F3F3F3Fu, mn_lo = r[2] & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (r[3] & 0x0F0F0F0Fu) | ((r[1] >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((r[3] >> 4) & 0x0F0F0F0Fu) | ((r[2] >> 2) & 0x30303030u);
+        float total = 0.f;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            float acc = 0.f;
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                const uint32_t qs = r[6 + 2 * (g >> 1) + m];
+                const uint32_t lo = (g & 1) ? ((qs >> 4) & 0x0F0F0F0Fu) : (qs & 0x0F0F0F0Fu);
+                const uint32_t hb = g < 4 ? ((r[4 + m] << (4 - g)) & 0x10101010u) : ((r[4 + m] >> (g - 4)) & 0x10101010u);
+                const uint32_t code = lo | hb;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc += ubyte_f(code, j) * xr[8 * g + 4 * m + j];
+            }
+            const float sc = ubyte_f(g < 4 ? sc_lo : sc_hi, g & 3), mn = ubyte_f(g < 4 ? mn_lo : mn_hi, g & 3);
+            total += (d * sc) * acc - (dmin * mn) * aux[g];
+        }
+        return total;
+    }
+};
+
+// ---- BF16 -----------------------------------------------------------------------------------
+template <> struct Unit64<QMOE_FMT_BF16> {
+    static constexpr int RAW = 32, AUX = 1;
+    static constexpr int ROW_ALIGN = 16;
+    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float*) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float4 v = load_x4(x, xdt, u * 64 + 4 * i);
+            xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+        }
+    }
+    __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
+        const uint4* p = (const uint4*)(row + (size_t)u * 128);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint4 v = p[i];
+            r[4 * i] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
+        }
+    }
+    __device__ __forceinline__ static float dot(const uint32_t* r, const float* xr, const float*) {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            s0 += __uint_as_float(r[i] << 16) * xr[2 * i];
+            s1 += __uint_as_float(r[i] & 0xFFFF0000u) * xr[2 * i + 1];
+        }
+        return s0 + s1;
+    }
+};
+
+// ---- problem lists ----------------------------------------------------------------------------
+static constexpr int STREAM_THREADS = 256;
+static constexpr int STREAM_WAVES = STREAM_THREADS / 64;
+static constexpr int STREAM_MAX_PROBLEMS = 16;
+
+struct StreamProblem {
+    const uint8_t* w;   // [n, k] packed rows
+    const uint8_t* w2;  // second matrix of a gate/up pair, or null
+    const void* x;      // one activation row
+    void* y;            // n outputs
+    int n, k;
+    int fmt, fmt2;
+    int xdt, ydt;
+    int first_item;     // worker that takes this problem's first row group (round robin across problems)
+    int xgroup;         // equal for consecutive problems that read the same activation row
+};
+
+struct StreamArgs {
+    int count;
+    int pad;
+    StreamProblem p[STREAM_MAX_PROBLEMS];
+};
+
+// True if (fmt, shape, alignment) can go through the streaming kernel.
+bool stream_supported(int fmt, const void* w, int n, int k, const void* x, int xdt);
+// Enqueue args.count (<= STREAM_MAX_PROBLEMS) supported problems as one launch.
+int stream_launch(StreamArgs& args, hipStream_t s);
+
+}  // namespace qmoe
