@@ -66,6 +66,18 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// acc + round(a * b): the product is rounded to fp32 before the add, never fused into an FMA
+// (the reference stores each routed product before accumulating it).
+__device__ __forceinline__ float add_product(float acc, float a, float b) {
+#pragma clang fp contract(off)
+    const float prod = a * b;
+    return acc + prod;
+}
+__device__ __forceinline__ float mul_unfused(float a, float b) {
+#pragma clang fp contract(off)
+    return a * b;
+}
+
 // g / (1 + exp(-g)) * u, the SwiGLU of mini_llm/ops/quantized_linear.py:367-370.
 __device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
 

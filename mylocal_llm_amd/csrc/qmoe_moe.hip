@@ -10,6 +10,7 @@
 //   hidden_act[A, F]  fp32 SwiGLU activations, terms[A, D] fp32 weighted expert outputs
 // with A = T*k.  Nothing is read back by the host.
 #include "qmoe_rowdot.hpp"
+#include "qmoe_stream.hpp"
 
 namespace qmoe {
 
@@ -180,7 +181,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
         for (int m = 0; m < MT; ++m) {
             float v = wave_sum(acc[m]);
             if (lane == m && j0 + m < cnt)
-                terms[(size_t)(lo + j0 + m) * d + row] = __fmul_rn(v, sorted_weight[lo + j0 + m]);
+                terms[(size_t)(lo + j0 + m) * d + row] = mul_unfused(v, sorted_weight[lo + j0 + m]);
         }
     }
 }
@@ -229,7 +230,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
             int p = order[s];
             if (p >= 0) acc = __fadd_rn(acc, terms[(size_t)p * d + i]);
         }
-        if (shared_out) acc = __fadd_rn(acc, __fmul_rn(shared_out[(size_t)t * d + i], sg));
+        if (shared_out) acc = add_product(acc, shared_out[(size_t)t * d + i], sg);
         store_out(out, odt, (size_t)t * d + i, acc);
     }
 }
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(256) void grouped_down_kernel(const void* const* __
     float v = wave_sum(acc[0]);
     if (lane == 0) {
         const int slot = slots ? slots[e] : e;
-        terms[(size_t)e * d + row] = __fmul_rn(v, routes[(int64_t)slot * route_stride]);
+        terms[(size_t)e * d + row] = mul_unfused(v, routes[(int64_t)slot * route_stride]);
     }
 }
 
@@ -292,7 +293,7 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MoeWorkspace {
     size_t weights, ids, offsets, active, n_active, status, sorted_token, sorted_weight, pos_of, hidden_act, terms,
-        shared_h, shared_out, total;
+        shared_h, shared_out, sig, problems, total;
 };
 
 static MoeWorkspace moe_layout(int tokens, int k, int n_experts, int d_model, int d_ff, int d_ff_shared) {
@@ -313,6 +314,8 @@ static MoeWorkspace moe_layout(int tokens, int k, int n_experts, int d_model, in
     w.terms = take(a * d_model * 4);
     w.shared_h = take((size_t)tokens * d_ff_shared * 4);
     w.shared_out = take((size_t)tokens * d_model * 4);
+    w.sig = take((size_t)tokens * 4);
+    w.problems = take(a * 64 + (size_t)tokens * 64);  // device-side problem list of the decode path
     w.total = at;
     return w;
 }
@@ -373,6 +376,13 @@ int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_b
         return fail(QMOE_EWORKSPACE, "%s: workspace must be 256-byte aligned and hold %zu bytes (got %zu)", who, L.total, workspace_bytes);
     char* ws = (char*)workspace;
     int rc;
+    static_assert(sizeof(StreamProblem) == 64, "problem list entries are 64 bytes");
+    if (decode_supported(a, ws + L.hidden_act)) {
+        DecodeBuffers db{(float*)(ws + L.weights), (int64_t*)(ws + L.ids), (int*)(ws + L.sorted_token),
+                         (float*)(ws + L.sorted_weight), (float*)(ws + L.sig), (int*)(ws + L.status),
+                         ws + L.problems, (int*)(ws + L.n_active), (float*)(ws + L.hidden_act), (float*)(ws + L.shared_h)};
+        return decode_launch(a, db, s);
+    }
     const float* weights = a.in_weights;
     const int64_t* ids = a.in_ids;
     if (a.logits) {
