@@ -175,12 +175,31 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup):
     hidden = torch.randn((tokens, d), device=device, generator=gen).to(torch.bfloat16)
     logits = torch.randn((n_banks, tokens, e), device=device, generator=gen)
     gate_vec = torch.randn(d, device=device, generator=gen) * 0.02
+    out = torch.empty((tokens, d), device=device, dtype=torch.bfloat16)
+    nbytes_ws = lib.qmoe_moe_workspace_bytes(tokens, k, e, d, f, fsh)
+    workspace = torch.empty(nbytes_ws, dtype=torch.uint8, device=device)
+    # the C ABI is the boundary: argument structs are built once, a step is one call
+    calls = []
+    for i in range(n_banks):
+        a = _lib.MoeArgs()
+        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), 2, tokens, k
+        a.logits, a.floor_value, a.renormalize = logits[i].data_ptr(), 2.0 ** -14, 1
+        banks[i].fill(a.bank)
+        g, u, dn = shareds[i]
+        a.shared_gate_w, a.shared_up_w, a.shared_down_w = g.data.data_ptr(), u.data.data_ptr(), dn.data.data_ptr()
+        a.shared_gate_fmt = a.shared_up_fmt = a.shared_down_fmt = _lib.FORMAT_ID[fmt]
+        a.d_ff_shared, a.shared_gate = fsh, gate_vec.data_ptr()
+        a.out, a.out_dtype = out.data_ptr(), 2
+        calls.append(a)
     state = {"i": 0}
+    wsp = ctypes.c_void_p(workspace.data_ptr())
 
-    def fn(_stream):
-        i = state["i"] % n_banks
+    def fn(stream):
+        a = calls[state["i"] % n_banks]
         state["i"] += 1
-        moe_step(hidden, banks[i], k, logits=logits[i], shared=shareds[i], shared_gate=gate_vec)
+        rc = lib.qmoe_moe_forward(ctypes.byref(a), wsp, nbytes_ws, stream)
+        if rc:
+            raise RuntimeError(lib.qmoe_last_error().decode())
 
     wall, ms = time_steps(torch, fn, steps, warmup)
     # algorithmic bytes: distinct selected experts (averaged over the banks' logits) + shared expert
@@ -204,6 +223,9 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device tensor copy (a kernel of known traffic, "
+                         "used to scale FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
@@ -218,6 +240,12 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     stream = LayerStream(torch, lib, "Q8_0", args.layers, 1, device)
     wall, ms = time_steps(torch, stream.step, args.steps, args.warmup)
     step_s = wall / args.steps
@@ -226,6 +254,11 @@ def main():
     launches = args.steps * stream.launches_per_step
     launch_ms = ms / launches
     achieved = stream.bytes_per_layer / (launch_ms * 1e-3) / 1e9
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "stream_q8_0_layer_m1_hbm_traffic.json")
+    if os.path.exists(traffic_file):  # from the two rocprofv3 --pmc runs described beside that file
+        with open(traffic_file) as fh:
+            traffic = json.load(fh).get("traffic_bytes_per_launch")
     result = {
         "metric": "effective weight GB/s (Q8_0 8B projections, M=1, 32 layers streamed)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -236,7 +269,7 @@ def main():
                    "weight_bytes_per_step": total_bytes, "tokens_per_s": round(1.0 / step_s, 1),
                    "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4), "activations": "fp32 N(0,1)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel": "linear (Q8_0, M=1), one layer = 7 projections per launch sequence",
                      "bytes_per_launch": stream.bytes_per_layer, "avg_launch_us": round(launch_ms * 1e3, 3)},
     }

@@ -45,46 +45,43 @@ struct DecodeRouteArgs {
 };
 
 __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs a) {
-    extern __shared__ float values[];  // n_experts floats when routing from logits
-    __shared__ float selected[32];
+    extern __shared__ uint32_t keys[];  // n_experts words when routing from logits
     __shared__ int64_t ids_sel[32];
     __shared__ float w_sel[32];
     __shared__ int order[32];
     const int t = blockIdx.x, lane = threadIdx.x;
     const int k = a.k;
+    // admission gate first: its loads are in flight while the row is routed
+    float adm = 0.f;
+    if (a.shared_gate) {
+        for (int i = 4 * lane; i < a.d; i += 256) {
+            const float4 hv = load_x4(a.hidden, a.xdt, t * a.d + i);
+            const float4 gv = *(const float4*)(a.shared_gate + i);
+            adm += (hv.x * gv.x + hv.y * gv.y) + (hv.z * gv.z + hv.w * gv.w);
+        }
+    }
     if (a.logits) {
-        router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, values, selected,
-                   w_sel, ids_sel);
+        router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, keys, w_sel, ids_sel);
     } else if (lane < k) {
         ids_sel[lane] = a.in_ids[(size_t)t * k + lane];
         w_sel[lane] = a.in_weights[(size_t)t * k + lane];
     }
     __syncthreads();
-    if (lane < k && a.out_weights) {
-        a.out_weights[(size_t)t * k + lane] = w_sel[lane];
-        a.out_ids[(size_t)t * k + lane] = ids_sel[lane];
-    }
-    if (lane == 0) {
-        // ascending expert id; equal ids keep slot order
-        for (int s = 0; s < k; ++s) {
-            int j = s;
-            while (j > 0 && ids_sel[order[j - 1]] > ids_sel[s]) { order[j] = order[j - 1]; --j; }
-            order[j] = s;
+    if (lane < k) {
+        if (a.out_weights) {
+            a.out_weights[(size_t)t * k + lane] = w_sel[lane];
+            a.out_ids[(size_t)t * k + lane] = ids_sel[lane];
         }
+        // rank of this selection in ascending expert id; equal ids keep slot order
+        const int64_t mine = ids_sel[lane];
+        int rank = 0;
+        for (int j = 0; j < k; ++j) rank += (ids_sel[j] < mine) || (ids_sel[j] == mine && j < lane);
+        order[rank] = lane;
     }
     __syncthreads();
-    // admission gate: sigmoid(hidden . g), evaluated without overflow
-    float adm = 0.f;
-    if (a.shared_gate) {
-        for (int i = lane; i < a.d; i += 64) {
-            const float hv = a.xdt == QMOE_DT_F32 ? Elem<QMOE_DT_F32>::load(a.hidden, (size_t)t * a.d + i)
-                           : a.xdt == QMOE_DT_F16 ? Elem<QMOE_DT_F16>::load(a.hidden, (size_t)t * a.d + i)
-                                                  : Elem<QMOE_DT_BF16>::load(a.hidden, (size_t)t * a.d + i);
-            adm += hv * a.shared_gate[i];
-        }
-        adm = wave_sum(adm);
-    }
+    if (a.shared_gate) adm = wave_sum(adm);
     if (lane == 0) {
+        // sigmoid(hidden . g) without overflow
         a.sig[t] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
         if (t == 0) *a.problem_count = a.tokens * (k + (a.shared_gate_w ? 1 : 0));
     }
@@ -131,17 +128,29 @@ __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs 
     }
 }
 
+static constexpr int LIST_STAGE = 48;  // problem descriptors held in LDS at a time
+
 // The streaming engine over a problem list that lives in device memory.
 template <int FMT, bool PAIR>
 __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const StreamProblem* __restrict__ list,
                                                                        const int* __restrict__ count) {
     __shared__ float partial[32 * 2 * 4];
+    __shared__ StreamProblem staged[LIST_STAGE];
     float xr[64], aux[8];
     int xgroup = -1;
     const int n = *count;
-    for (int i = 0; i < n; ++i) {
-        const StreamProblem p = list[i];
-        if (p.n > 0) stream_dispatch_shape<FMT, PAIR>(p, partial, xr, aux, xgroup);
+    // descriptors are fetched a stage at a time by the whole workgroup, not one dependent
+    // load per problem
+    for (int base = 0; base < n; base += LIST_STAGE) {
+        const int m = n - base < LIST_STAGE ? n - base : LIST_STAGE;
+        __syncthreads();
+        const uint4* src = (const uint4*)(list + base);
+        uint4* dst = (uint4*)staged;
+        for (int i = threadIdx.x; i < m * 4; i += STREAM_THREADS) dst[i] = src[i];
+        __syncthreads();
+        for (int i = 0; i < m; ++i) {
+            if (staged[i].n > 0) stream_dispatch_shape<FMT, PAIR>(staged[i], partial, xr, aux, xgroup);
+        }
     }
 }
 
@@ -179,9 +188,10 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
     const int shared_parts = a.shared_down ? a.fsh >> 7 : 0;
     const bool routed = lane < k * LPE;
     const bool shared = lane >= 48 && lane - 48 < shared_parts;
-    int slot = routed ? lane / LPE : 0;
+    const int slot = routed ? lane / LPE : 0;
     const int part = routed ? lane % LPE : (shared ? lane - 48 : 0);
     const int e = routed ? a.sorted_ids[(size_t)t * k + slot] : 0;
+    const float route_w = lane < k ? a.sorted_w[(size_t)t * k + lane] : 0.f;  // lane j holds weight j
     const bool live = (routed && e >= 0) || shared;
     const int kk = shared ? a.fsh : a.f;
     const int64_t rbytes = row_bytes_dev(FMT, kk);
@@ -216,7 +226,8 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
         float acc = 0.f;
         for (int j = 0; j < k; ++j) {
             const float yj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(yr), j * LPE));
-            acc = add_product(acc, yj, a.sorted_w[(size_t)t * k + j]);
+            const float wj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(route_w), j));
+            acc = add_product(acc, yj, wj);
         }
         if (a.shared_down) {
             const float y63 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ys), 63));

@@ -9,9 +9,8 @@ namespace qmoe {
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ logits, int n, int k,
                                                          float floor_value, int renorm,
                                                          float* __restrict__ weights, int64_t* __restrict__ ids) {
-    extern __shared__ float values[];
-    __shared__ float selected[32];
-    router_row(logits + (size_t)blockIdx.x * n, n, k, floor_value, renorm, values, selected,
+    extern __shared__ uint32_t keys[];
+    router_row(logits + (size_t)blockIdx.x * n, n, k, floor_value, renorm, keys,
                weights + (size_t)blockIdx.x * k, ids + (size_t)blockIdx.x * k);
 }
 
