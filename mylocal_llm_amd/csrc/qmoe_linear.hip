@@ -137,6 +137,7 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
         args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, fmt, xdt, ydt, 0, 0};
         return stream_launch(args, s);
     }
+    if (smallm_supported(fmt, w, n, k, x, xdt, tokens)) return smallm_launch(fmt, w, n, k, x, xdt, tokens, y, ydt, s);
     const bool fast = rows_fast(fmt, w, row_bytes(fmt, k), k) && x_fast(x, xdt, k);
     if (xdt == QMOE_DT_F32) launch_linear_mt<QMOE_DT_F32>(w, fmt, n, k, fast, x, tokens, y, ydt, s);
     else if (xdt == QMOE_DT_F16) launch_linear_mt<QMOE_DT_F16>(w, fmt, n, k, fast, x, tokens, y, ydt, s);

@@ -85,6 +85,18 @@ template <> struct Unit64<QMOE_FMT_Q8_0> {
         }
         return d0 * s0 + d1 * s1;
     }
+    // the 64 dequantised weights of the unit, in unit order
+    __device__ __forceinline__ static void decode(const uint32_t* r, float* w) {
+        const float d0 = half_bits_to_float(r[0] & 0xFFFFu), d1 = half_bits_to_float(r[8] >> 16);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const int b0 = 2 + i, b1 = 36 + i;
+            w[i] = d0 * sbyte(r[b0 >> 2], b0 & 3);
+            w[32 + i] = d1 * sbyte(r[b1 >> 2], b1 & 3);
+        }
+    }
+    // column of unit element 8*m (elements 8m..8m+7 are consecutive columns)
+    __device__ __forceinline__ static int kstep(int u, int m) { return u * 64 + 8 * m; }
 };
 
 // ---- Q6_K -----------------------------------------------------------------------------------
@@ -142,6 +154,25 @@ template <> struct Unit64<QMOE_FMT_Q6_K> {
         }
         return total;
     }
+    __device__ __forceinline__ static void decode(const uint32_t* r, float* w) {
+        const float d = half_bits_to_float(r[14]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float scale = d * sbyte(r[12 + (q >> 1)], q & 1);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const uint32_t src = (q & 1) ? r[4 + m] : r[m];
+                const uint32_t lo = (q & 2) ? ((src >> 4) & 0x0F0F0F0Fu) : (src & 0x0F0F0F0Fu);
+                const uint32_t hi = (r[8 + m] >> (2 * q)) & 0x03030303u;
+                const uint32_t code = lo | (hi << 4);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[16 * q + 4 * m + j] = scale * (ubyte_f(code, j) - 32.0f);
+            }
+        }
+    }
+    __device__ __forceinline__ static int kstep(int u, int m) {
+        return (u >> 2) * 256 + ((u >> 1) & 1) * 128 + (u & 1) * 16 + 32 * (m >> 1) + 8 * (m & 1);
+    }
 };
 
 // ---- Q5_K -----------------------------------------------------------------------------------
@@ -197,6 +228,27 @@ template <> struct Unit64<QMOE_FMT_Q5_K> {
         }
         return total;
     }
+    __device__ __forceinline__ static void decode(const uint32_t* r, float* w) {
+        const float d = half_bits_to_float(r[0] & 0xFFFFu), dmin = half_bits_to_float(r[0] >> 16);
+        const uint32_t sc_lo = r[1] & 0x3F3F3F3Fu, mn_lo = r[2] & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (r[3] & 0x0F0F0F0Fu) | ((r[1] >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((r[3] >> 4) & 0x0F0F0F0Fu) | ((r[2] >> 2) & 0x30303030u);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            const float scale = d * ubyte_f(g < 4 ? sc_lo : sc_hi, g & 3);
+            const float floor_ = dmin * ubyte_f(g < 4 ? mn_lo : mn_hi, g & 3);
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                const uint32_t qs = r[6 + 2 * (g >> 1) + m];
+                const uint32_t lo = (g & 1) ? ((qs >> 4) & 0x0F0F0F0Fu) : (qs & 0x0F0F0F0Fu);
+                const uint32_t hb = g < 4 ? ((r[4 + m] << (4 - g)) & 0x10101010u) : ((r[4 + m] >> (g - 4)) & 0x10101010u);
+                const uint32_t code = lo | hb;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[8 * g + 4 * m + j] = scale * ubyte_f(code, j) - floor_;
+            }
+        }
+    }
+    __device__ __forceinline__ static int kstep(int u, int m) { return (u >> 2) * 256 + (u & 3) * 8 + 32 * m; }
 };
 
 // ---- BF16 -----------------------------------------------------------------------------------
@@ -227,6 +279,14 @@ template <> struct Unit64<QMOE_FMT_BF16> {
         }
         return s0 + s1;
     }
+    __device__ __forceinline__ static void decode(const uint32_t* r, float* w) {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            w[2 * i] = __uint_as_float(r[i] << 16);
+            w[2 * i + 1] = __uint_as_float(r[i] & 0xFFFF0000u);
+        }
+    }
+    __device__ __forceinline__ static int kstep(int u, int m) { return u * 64 + 8 * m; }
 };
 
 // ---- problem lists ----------------------------------------------------------------------------
@@ -378,6 +438,11 @@ bool stream_supported(int fmt, const void* w, int n, int k, const void* x, int x
 int stream_launch(StreamArgs& args, hipStream_t s);
 
 int stream_grid();
+
+// ---- small-batch MFMA linear (qmoe_smallm.hip) ------------------------------------------------
+bool smallm_supported(int fmt, const void* w, int n, int k, const void* x, int xdt, int tokens);
+int smallm_launch(int fmt, const void* w, int n, int k, const void* x, int xdt, int tokens, void* y, int ydt,
+                  hipStream_t s);
 
 // ---- decode-time MoE step (qmoe_decode.hip) -----------------------------------------------------
 struct DecodeBuffers {  // workspace regions, all device pointers

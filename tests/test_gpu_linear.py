@@ -28,8 +28,11 @@ def test_linear_matches_oracle(cuda, fmt, m):
     want = R.linear(x, *triple(w))
     got = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
     assert got.shape == (m, 96) and got.dtype == np.float32
-    assert rel_l2(got, want) <= 2e-6 <= REL_L2
-    np.testing.assert_allclose(got, native.c_linear(x, *triple(w)), rtol=2e-5, atol=2e-5 * np.abs(want).max())
+    # more than one token runs on MFMA with weights and fp32 activations each split into two
+    # bf16 terms (16 significant bits): still two orders of magnitude inside the 1e-3 bar
+    tol = 2e-5 if m > 1 else 2e-6
+    assert rel_l2(got, want) <= tol <= REL_L2
+    np.testing.assert_allclose(got, native.c_linear(x, *triple(w)), rtol=10 * tol, atol=10 * tol * np.abs(want).max())
 
 
 def test_config0_single_q8_0_matrix_batch1(cuda):
@@ -78,7 +81,8 @@ def test_linear_low_precision_activations(cuda, dtype, tol, fmt):
     got = quantized_linear(x.to(cuda), upload(w, cuda))
     assert got.dtype == dtype
     want_rounded = torch.from_numpy(want).to(dtype).float().numpy()
-    assert np.abs(got.float().cpu().numpy() - want_rounded).max() <= tol
+    # one rounding to the output type: within an ulp of the rounded oracle value
+    assert np.abs(got.float().cpu().numpy() - want_rounded).max() <= tol * max(1.0, float(np.abs(want).max()))
     assert rel_l2(got.float().cpu().numpy(), want) <= (5e-3 if dtype == torch.bfloat16 else 1e-3)
 
 
@@ -154,7 +158,7 @@ def test_packed_expert_matches_oracle(cuda, fmts, fuse):
     want = R.expert_ffn(x, triple(gate), triple(up), triple(down))
     expert = PackedExpertFFNInference(upload(gate, cuda), upload(up, cuda), upload(down, cuda), fuse_gate_up=fuse)
     got = expert.forward(torch.from_numpy(x).to(cuda)).cpu().numpy()
-    assert rel_l2(got, want) <= 1e-5 <= REL_L2
+    assert rel_l2(got, want) <= 5e-5 <= REL_L2  # three tokens: MFMA path, 16-bit operand splits
     with pytest.raises(ValueError, match="transposed"):
         PackedExpertFFNInference(expert.gate, expert.up, expert.gate)
 
@@ -186,9 +190,9 @@ def test_8b_projection_shapes_linearity_and_row_checks(cuda, fmt, shape):
     combo = torch.from_numpy((0.5 * x[0] - 0.25 * x[1])[None]).to(cuda)
     yc = quantized_linear(combo, dev)
     lin = 0.5 * y[0] - 0.25 * y[1]
-    assert rel_l2(yc[0].cpu().numpy(), lin.cpu().numpy()) <= 1e-5
+    assert rel_l2(yc[0].cpu().numpy(), lin.cpu().numpy()) <= 3e-5
     rows = rng.choice(n, 24, replace=False)
     sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), fmt)
     want = R.linear(x, *triple(sub))
     got = y.cpu().numpy()[:, rows]
-    assert rel_l2(got, want) <= 2e-6
+    assert rel_l2(got, want) <= 3e-5  # two tokens: MFMA path, 16-bit operand splits
