@@ -136,8 +136,9 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
                                                                        const int* __restrict__ count) {
     __shared__ float partial[32 * 2 * 4];
     __shared__ StreamProblem staged[LIST_STAGE];
+    __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     float xr[64], aux[8];
-    int xgroup = -1;
+    int xgroup = -1, xstaged = -1;
     const int n = *count;
     // descriptors are fetched a stage at a time by the whole workgroup, not one dependent
     // load per problem
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
         for (int i = threadIdx.x; i < m * 4; i += STREAM_THREADS) dst[i] = src[i];
         __syncthreads();
         for (int i = 0; i < m; ++i) {
-            if (staged[i].n > 0) stream_dispatch_shape<FMT, PAIR>(staged[i], partial, xr, aux, xgroup);
+            if (staged[i].n > 0) stream_dispatch_shape<FMT, PAIR>(staged[i], partial, xs, xstaged, xr, aux, xgroup);
         }
     }
 }
@@ -208,8 +209,8 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
         U::load_w(rp, 2 * part + 1, ra[r][1]);
     }
     float x0[64], x1[64], aux0[U::AUX], aux1[U::AUX];
-    U::load_x(xsrc, QMOE_DT_F32, 2 * part, x0, aux0);
-    U::load_x(xsrc, QMOE_DT_F32, 2 * part + 1, x1, aux1);
+    U::load_x(GlobalX{xsrc, QMOE_DT_F32}, 2 * part, x0, aux0);
+    U::load_x(GlobalX{xsrc, QMOE_DT_F32}, 2 * part + 1, x1, aux1);
     if (!live) {
 #pragma unroll
         for (int i = 0; i < 64; ++i) { x0[i] = 0.f; x1[i] = 0.f; }

@@ -15,9 +15,10 @@ namespace qmoe {
 template <int FMT, bool PAIR>
 __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamArgs args) {
     __shared__ float partial[32 * 2 * 4];
+    __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     float xr[64], aux[8];
-    int xgroup = -1;
-    for (int i = 0; i < args.count; ++i) stream_dispatch_shape<FMT, PAIR>(args.p[i], partial, xr, aux, xgroup);
+    int xgroup = -1, staged = -1;
+    for (int i = 0; i < args.count; ++i) stream_dispatch_shape<FMT, PAIR>(args.p[i], partial, xs, staged, xr, aux, xgroup);
 }
 
 // ---- host side ---------------------------------------------------------------------------------

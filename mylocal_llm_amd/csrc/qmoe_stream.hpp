@@ -52,16 +52,30 @@ __device__ __forceinline__ float4 load_x4(const void* x, int xdt, int i) {
     return Elem<QMOE_DT_BF16>::load4(x, i);
 }
 
+// Where a lane's activation values come from: global memory of any supported type, or the
+// workgroup's fp32 staging area in LDS.  The staging area carries 4 floats of padding after
+// every 64, so that lanes reading consecutive units (272 bytes apart) spread over all banks.
+struct GlobalX {
+    const void* x;
+    int xdt;
+    __device__ __forceinline__ float4 operator()(int i) const { return load_x4(x, xdt, i); }
+};
+struct StagedX {
+    const float* xs;
+    __device__ __forceinline__ static int at(int i) { return i + 4 * (i >> 6); }
+    __device__ __forceinline__ float4 operator()(int i) const { return *(const float4*)(xs + at(i)); }
+};
+
 template <int FMT> struct Unit64;
 
 // ---- Q8_0 -----------------------------------------------------------------------------------
 template <> struct Unit64<QMOE_FMT_Q8_0> {
     static constexpr int RAW = 17, AUX = 1;
     static constexpr int ROW_ALIGN = 4;
-    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float*) {
+    template <class X> __device__ __forceinline__ static void load_x(const X& x, int u, float* xr, float*) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            float4 v = load_x4(x, xdt, u * 64 + 4 * i);
+            float4 v = x(u * 64 + 4 * i);
             xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
         }
     }
@@ -105,14 +119,14 @@ template <> struct Unit64<QMOE_FMT_Q8_0> {
 template <> struct Unit64<QMOE_FMT_Q6_K> {
     static constexpr int RAW = 15, AUX = 4;
     static constexpr int ROW_ALIGN = 2;
-    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float* aux) {
+    template <class X> __device__ __forceinline__ static void load_x(const X& x, int u, float* xr, float* aux) {
         const int base = (u >> 2) * 256 + ((u >> 1) & 1) * 128 + (u & 1) * 16;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             float s = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float4 v = load_x4(x, xdt, base + 32 * q + 4 * i);
+                float4 v = x(base + 32 * q + 4 * i);
                 xr[16 * q + 4 * i] = v.x; xr[16 * q + 4 * i + 1] = v.y; xr[16 * q + 4 * i + 2] = v.z; xr[16 * q + 4 * i + 3] = v.w;
                 s += (v.x + v.y) + (v.z + v.w);
             }
@@ -181,11 +195,11 @@ template <> struct Unit64<QMOE_FMT_Q6_K> {
 template <> struct Unit64<QMOE_FMT_Q5_K> {
     static constexpr int RAW = 14, AUX = 8;
     static constexpr int ROW_ALIGN = 16;
-    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float* aux) {
+    template <class X> __device__ __forceinline__ static void load_x(const X& x, int u, float* xr, float* aux) {
         const int base = (u >> 2) * 256 + (u & 3) * 8;
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            float4 a = load_x4(x, xdt, base + 32 * g), b = load_x4(x, xdt, base + 32 * g + 4);
+            float4 a = x(base + 32 * g), b = x(base + 32 * g + 4);
             xr[8 * g] = a.x; xr[8 * g + 1] = a.y; xr[8 * g + 2] = a.z; xr[8 * g + 3] = a.w;
             xr[8 * g + 4] = b.x; xr[8 * g + 5] = b.y; xr[8 * g + 6] = b.z; xr[8 * g + 7] = b.w;
             aux[g] = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
@@ -255,10 +269,10 @@ template <> struct Unit64<QMOE_FMT_Q5_K> {
 template <> struct Unit64<QMOE_FMT_BF16> {
     static constexpr int RAW = 32, AUX = 1;
     static constexpr int ROW_ALIGN = 16;
-    __device__ __forceinline__ static void load_x(const void* x, int xdt, int u, float* xr, float*) {
+    template <class X> __device__ __forceinline__ static void load_x(const X& x, int u, float* xr, float*) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            float4 v = load_x4(x, xdt, u * 64 + 4 * i);
+            float4 v = x(u * 64 + 4 * i);
             xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
         }
     }
@@ -293,6 +307,8 @@ template <> struct Unit64<QMOE_FMT_BF16> {
 static constexpr int STREAM_THREADS = 256;
 static constexpr int STREAM_WAVES = STREAM_THREADS / 64;
 static constexpr int STREAM_MAX_PROBLEMS = 16;
+static constexpr int STREAM_MAX_K = 16384;  // activations of one problem staged in LDS as fp32
+static constexpr int STREAM_XS_FLOATS = STREAM_MAX_K + 4 * (STREAM_MAX_K / 64);
 
 struct StreamProblem {
     const uint8_t* w;   // [n, k] packed rows
@@ -331,8 +347,8 @@ template <int FMT, bool PAIR> struct RowRegs {
 // Rows of `LR` lanes each (64/LR rows per wave and step); WR waves share one row; PD rows
 // are requested ahead of the one being reduced.
 template <int FMT, bool PAIR, int LR, int WR, int PD>
-__device__ __forceinline__ void stream_problem(const StreamProblem& p, float* partial, float (&xr)[64], float (&aux)[8],
-                                               int& xgroup) {
+__device__ __forceinline__ void stream_problem(const StreamProblem& p, float* partial, float* xs, int& staged,
+                                               float (&xr)[64], float (&aux)[8], int& xgroup) {
     using U = Unit64<FMT>;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int units = p.k >> 6;
@@ -347,7 +363,7 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
     const int workers = WR > 1 ? gridDim.x : gridDim.x * STREAM_WAVES;
     const int me = WR > 1 ? blockIdx.x : blockIdx.x * STREAM_WAVES + wave;
     int item = (me - p.first_item + workers) % workers;
-    if (item >= items) return;
+    const bool busy = item < items;
 
     RowRegs<FMT, PAIR> buf[PD + 1];
     auto fetch = [&](RowRegs<FMT, PAIR>& r, int it) {
@@ -359,10 +375,19 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
 #pragma unroll
     for (int j = 0; j < PD; ++j)
         if (item + j * workers < items) fetch(buf[j], item + j * workers);
+    // New activations are staged once per workgroup in LDS (as fp32) while this wave's first
+    // rows are already in flight; every wave of the workgroup passes here for every problem.
+    if (staged != p.xgroup) {
+        __syncthreads();
+        for (int i = 4 * threadIdx.x; i < p.k; i += 4 * STREAM_THREADS) *(float4*)(xs + StagedX::at(i)) = load_x4(p.x, p.xdt, i);
+        __syncthreads();
+        staged = p.xgroup;
+    }
+    if (!busy) return;
     // The activation slice of the lane's unit position stays in registers across problems
     // that read the same activations (xgroup names what is loaded).
     if (xgroup != p.xgroup) {
-        U::load_x(p.x, p.xdt, uu, xr, aux);
+        U::load_x(StagedX{xs}, uu, xr, aux);
         if (!active) {
 #pragma unroll
             for (int i = 0; i < 64; ++i) xr[i] = 0.f;
@@ -419,17 +444,17 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
 }
 
 template <int FMT, bool PAIR>
-__device__ __forceinline__ void stream_dispatch_shape(const StreamProblem& p, float* partial, float (&xr)[64],
-                                                      float (&aux)[8], int& xgroup) {
+__device__ __forceinline__ void stream_dispatch_shape(const StreamProblem& p, float* partial, float* xs, int& staged,
+                                                      float (&xr)[64], float (&aux)[8], int& xgroup) {
     const int units = p.k >> 6;
     // rows requested ahead: bounded by the 256-VGPR budget (a BF16 unit is 32 dwords per row)
     constexpr int PD = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (PAIR ? 1 : 2);
-    if (units <= 8) stream_problem<FMT, PAIR, 8, 1, PD>(p, partial, xr, aux, xgroup);
-    else if (units <= 16) stream_problem<FMT, PAIR, 16, 1, PD>(p, partial, xr, aux, xgroup);
-    else if (units <= 32) stream_problem<FMT, PAIR, 32, 1, PD>(p, partial, xr, aux, xgroup);
-    else if (units <= 64) stream_problem<FMT, PAIR, 64, 1, PD>(p, partial, xr, aux, xgroup);
-    else if (units <= 128) stream_problem<FMT, PAIR, 64, 2, PD>(p, partial, xr, aux, xgroup);
-    else stream_problem<FMT, PAIR, 64, 4, PD>(p, partial, xr, aux, xgroup);
+    if (units <= 8) stream_problem<FMT, PAIR, 8, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
+    else if (units <= 16) stream_problem<FMT, PAIR, 16, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
+    else if (units <= 32) stream_problem<FMT, PAIR, 32, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
+    else if (units <= 64) stream_problem<FMT, PAIR, 64, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
+    else if (units <= 128) stream_problem<FMT, PAIR, 64, 2, PD>(p, partial, xs, staged, xr, aux, xgroup);
+    else stream_problem<FMT, PAIR, 64, 4, PD>(p, partial, xs, staged, xr, aux, xgroup);
 }
 
 // True if (fmt, shape, alignment) can go through the streaming kernel.
