@@ -18,6 +18,7 @@
 namespace qmoe {
 
 static constexpr int DECODE_MAX_TOKENS = 16;
+static constexpr int LIST_STAGE = 48;  // problem descriptors held in LDS at a time
 // rows of the output one wave produces in the down kernel (a BF16 unit needs twice the registers)
 template <int FMT> struct DownRows { static constexpr int PER_WAVE = FMT == QMOE_FMT_BF16 ? 1 : 2; };
 
@@ -44,24 +45,34 @@ struct DecodeRouteArgs {
     int renorm, n_experts, k, d, f, fsh, fmt, xdt, tokens, workers;
 };
 
+// This lane's part of hidden[t] . g; the loads of eight steps travel together.
+__device__ __forceinline__ float admission_partial(const void* hidden, int xdt, int t, int d, const float* g, int lane) {
+    float acc = 0.f;
+    for (int base = 0; base < d; base += 2048) {
+        float4 hv[8], gv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = base + 4 * lane + 256 * j;
+            const bool in = i < d;
+            hv[j] = in ? load_x4(hidden, xdt, t * d + i) : make_float4(0, 0, 0, 0);
+            gv[j] = in ? *(const float4*)(g + i) : make_float4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += (hv[j].x * gv[j].x + hv[j].y * gv[j].y) + (hv[j].z * gv[j].z + hv[j].w * gv[j].w);
+    }
+    return acc;
+}
+
 __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs a) {
-    extern __shared__ uint32_t keys[];  // n_experts words when routing from logits
     __shared__ int64_t ids_sel[32];
     __shared__ float w_sel[32];
     __shared__ int order[32];
     const int t = blockIdx.x, lane = threadIdx.x;
     const int k = a.k;
     // admission gate first: its loads are in flight while the row is routed
-    float adm = 0.f;
-    if (a.shared_gate) {
-        for (int i = 4 * lane; i < a.d; i += 256) {
-            const float4 hv = load_x4(a.hidden, a.xdt, t * a.d + i);
-            const float4 gv = *(const float4*)(a.shared_gate + i);
-            adm += (hv.x * gv.x + hv.y * gv.y) + (hv.z * gv.z + hv.w * gv.w);
-        }
-    }
+    float adm = a.shared_gate ? admission_partial(a.hidden, a.xdt, t, a.d, a.shared_gate, lane) : 0.f;
     if (a.logits) {
-        router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, keys, w_sel, ids_sel);
+        router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w_sel, ids_sel);
     } else if (lane < k) {
         ids_sel[lane] = a.in_ids[(size_t)t * k + lane];
         w_sel[lane] = a.in_weights[(size_t)t * k + lane];
@@ -98,7 +109,6 @@ __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs 
         p.x = (const uint8_t*)a.hidden + (size_t)t * xbytes;
         p.k = a.d;
         p.fmt = a.fmt;
-        p.fmt2 = a.fmt;
         p.xdt = a.xdt;
         p.ydt = QMOE_DT_F32;
         p.xgroup = t;
@@ -123,12 +133,16 @@ __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs 
             p.n = a.fsh;
             cursor = token_cursor + (long)k * items_r * (units > 64 ? STREAM_WAVES : 1);
         }
-        p.first_item = units > 64 ? (int)((cursor / STREAM_WAVES) % (a.workers / STREAM_WAVES)) : (int)(cursor % a.workers);
+        if (units > 64) {
+            p.first_item = (int)((cursor / STREAM_WAVES) % (a.workers / STREAM_WAVES));
+            p.flat_end = 0;
+        } else {
+            p.first_item = (int)cursor;
+            p.flat_end = (int)cursor + (lane < k ? items_r : items_s);
+        }
         a.problems[(size_t)t * per_token + lane] = p;
     }
 }
-
-static constexpr int LIST_STAGE = 48;  // problem descriptors held in LDS at a time
 
 // The streaming engine over a problem list that lives in device memory.
 template <int FMT, bool PAIR>
@@ -137,8 +151,6 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
     __shared__ float partial[32 * 2 * 4];
     __shared__ StreamProblem staged[LIST_STAGE];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
-    float xr[64], aux[8];
-    int xgroup = -1, xstaged = -1;
     const int n = *count;
     // descriptors are fetched a stage at a time by the whole workgroup, not one dependent
     // load per problem
@@ -149,10 +161,107 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
         uint4* dst = (uint4*)staged;
         for (int i = threadIdx.x; i < m * 4; i += STREAM_THREADS) dst[i] = src[i];
         __syncthreads();
-        for (int i = 0; i < m; ++i) {
-            if (staged[i].n > 0) stream_dispatch_shape<FMT, PAIR>(staged[i], partial, xs, xstaged, xr, aux, xgroup);
+        // the stage's share of the flat item stream (empty when the rows are wider than a wave)
+        const int wide = (staged[0].k >> 6) > 64;
+        stream_run<FMT, PAIR>(staged, m, wide ? 0 : staged[0].first_item, wide ? 0 : staged[m - 1].flat_end, partial, xs);
+    }
+}
+
+// Routing fused into the gate/up launch (up to FUSED_MAX_TOKENS tokens): every workgroup
+// routes the tokens itself (its four waves share them), so the problem list never leaves
+// LDS and no launch sits between the logits and the first expert byte.  Workgroup 0 also
+// publishes the routing for the down kernel.
+static constexpr int FUSED_MAX_TOKENS = 4;
+
+template <int FMT>
+__global__ __launch_bounds__(STREAM_THREADS, 2) void decode_pairs_fused_kernel(const DecodeRouteArgs a) {
+    __shared__ float partial[32 * 2 * 4];
+    __shared__ StreamProblem staged[LIST_STAGE];
+    __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
+    __shared__ int64_t ids_sel[FUSED_MAX_TOKENS][32];
+    __shared__ float w_sel[FUSED_MAX_TOKENS][32];
+    __shared__ int order[FUSED_MAX_TOKENS][32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int k = a.k, tokens = a.tokens;
+    for (int t = wave; t < tokens; t += STREAM_WAVES) {
+        const float adm_part = a.shared_gate ? admission_partial(a.hidden, a.xdt, t, a.d, a.shared_gate, lane) : 0.f;
+        float adm = adm_part;
+        if (a.logits) {
+            router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w_sel[t], ids_sel[t]);
+        } else if (lane < k) {
+            ids_sel[t][lane] = a.in_ids[(size_t)t * k + lane];
+            w_sel[t][lane] = a.in_weights[(size_t)t * k + lane];
+        }
+        if (a.shared_gate) adm = wave_sum(adm);
+        if (blockIdx.x == 0 && lane == 0)
+            a.sig[t] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < tokens * k) {
+        const int t = threadIdx.x / k, s = threadIdx.x % k;
+        const int64_t mine = ids_sel[t][s];
+        int rank = 0;
+        for (int j = 0; j < k; ++j) rank += (ids_sel[t][j] < mine) || (ids_sel[t][j] == mine && j < s);
+        order[t][rank] = s;
+        if (blockIdx.x == 0 && a.out_weights) {
+            a.out_weights[(size_t)t * k + s] = w_sel[t][s];
+            a.out_ids[(size_t)t * k + s] = mine;
         }
     }
+    __syncthreads();
+    const int per_token = k + (a.shared_gate_w ? 1 : 0);
+    const int count = tokens * per_token;
+    if ((int)threadIdx.x < count) {
+        const int t = threadIdx.x / per_token, j = threadIdx.x % per_token;
+        const int units = a.d >> 6;
+        const int lr = units <= 8 ? 8 : units <= 16 ? 16 : units <= 32 ? 32 : 64;
+        const int rpw = 64 / lr;
+        const int items_r = (a.f + rpw - 1) / rpw, items_s = a.shared_gate_w ? (a.fsh + rpw - 1) / rpw : 0;
+        const int wide = units > 64 ? STREAM_WAVES : 1;
+        const int64_t xbytes = (int64_t)a.d * (a.xdt == QMOE_DT_F32 ? 4 : 2);
+        const long token_cursor = (long)t * ((long)k * items_r + items_s) * wide;
+        StreamProblem p;
+        p.x = (const uint8_t*)a.hidden + (size_t)t * xbytes;
+        p.k = a.d;
+        p.fmt = a.fmt;
+        p.xdt = a.xdt;
+        p.ydt = QMOE_DT_F32;
+        p.xgroup = t;
+        long cursor;
+        if (j < k) {
+            const int s = order[t][j];
+            const int64_t e = ids_sel[t][s];
+            const bool ok = e >= 0 && e < a.n_experts;
+            const int64_t ee = ok ? e : 0;
+            p.w = a.gate + ee * a.gate_stride;
+            p.w2 = a.up + ee * a.up_stride;
+            p.y = a.h + ((size_t)t * k + j) * a.f;
+            p.n = ok ? a.f : 0;
+            if (blockIdx.x == 0) {
+                if (!ok) *a.status = 1;
+                a.sorted_ids[(size_t)t * k + j] = ok ? (int)e : -1;
+                a.sorted_w[(size_t)t * k + j] = w_sel[t][s];
+            }
+            cursor = token_cursor + (long)j * items_r * wide;
+        } else {
+            p.w = a.shared_gate_w;
+            p.w2 = a.shared_up_w;
+            p.y = a.hs + (size_t)t * a.fsh;
+            p.n = a.fsh;
+            cursor = token_cursor + (long)k * items_r * wide;
+        }
+        if (units > 64) {
+            p.first_item = (int)((cursor / STREAM_WAVES) % (a.workers / STREAM_WAVES));
+            p.flat_end = 0;
+        } else {
+            p.first_item = (int)cursor;
+            p.flat_end = (int)cursor + (j < k ? items_r : items_s);
+        }
+        staged[threadIdx.x] = p;
+    }
+    __syncthreads();
+    const int wide = (a.d >> 6) > 64;
+    stream_run<FMT, true>(staged, count, 0, wide ? 0 : staged[count - 1].flat_end, partial, xs);
 }
 
 template <int LPE>
@@ -308,9 +417,20 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     r.xdt = a.hidden_dtype;
     r.tokens = a.tokens;
     r.workers = grid * STREAM_WAVES;
-    hipLaunchKernelGGL(decode_route_kernel, dim3(a.tokens), dim3(64), a.logits ? (size_t)b.n_experts * 4 : 0, s, r);
-    int rc = check_launch("qmoe_moe_forward(route)");
-    if (rc) return rc;
+    int rc;
+    const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.tokens * (a.top_k + 1) <= LIST_STAGE;
+    if (fused) {
+        const dim3 fg(grid), fb(STREAM_THREADS);
+        switch (b.gate_fmt) {
+        case QMOE_FMT_Q8_0: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q8_0>, fg, fb, 0, s, r); break;
+        case QMOE_FMT_Q6_K: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q6_K>, fg, fb, 0, s, r); break;
+        case QMOE_FMT_Q5_K: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q5_K>, fg, fb, 0, s, r); break;
+        default: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_BF16>, fg, fb, 0, s, r); break;
+        }
+        if ((rc = check_launch("qmoe_moe_forward(route + gate/up)"))) return rc;
+    } else {
+    hipLaunchKernelGGL(decode_route_kernel, dim3(a.tokens), dim3(64), 0, s, r);
+    if ((rc = check_launch("qmoe_moe_forward(route)"))) return rc;
 #define QMOE_LIST(F) hipLaunchKernelGGL((stream_list_kernel<F, true>), dim3(grid), dim3(STREAM_THREADS), 0, s, \
                                         (const StreamProblem*)w.problems, (const int*)w.problem_count)
     switch (b.gate_fmt) {
@@ -321,6 +441,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     }
 #undef QMOE_LIST
     if ((rc = check_launch("qmoe_moe_forward(gate/up)"))) return rc;
+    }
     DecodeDownArgs d{};
     d.down = (const uint8_t*)b.down;
     d.down_stride = b.down_stride;

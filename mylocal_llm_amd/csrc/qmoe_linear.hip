@@ -134,7 +134,7 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
     if (tokens == 1 && stream_supported(fmt, w, n, k, x, xdt)) {
         StreamArgs args{};
         args.count = 1;
-        args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, fmt, xdt, ydt, 0, 0};
+        args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, 0, xdt, ydt, 0, 0};
         return stream_launch(args, s);
     }
     if (smallm_supported(fmt, w, n, k, x, xdt, tokens)) return smallm_launch(fmt, w, n, k, x, xdt, tokens, y, ydt, s);
@@ -197,7 +197,7 @@ int swiglu_impl(const void* gate, int gf, const void* up, int uf, int f, int k, 
     if (tokens == 1 && gf == uf && stream_supported(gf, gate, f, k, x, xdt) && stream_supported(uf, up, f, k, x, xdt)) {
         StreamArgs args{};
         args.count = 1;
-        args.p[0] = StreamProblem{(const uint8_t*)gate, (const uint8_t*)up, x, h, f, k, gf, uf, xdt, hdt, 0, 0};
+        args.p[0] = StreamProblem{(const uint8_t*)gate, (const uint8_t*)up, x, h, f, k, gf, 0, xdt, hdt, 0, 0};
         return stream_launch(args, s);
     }
     const bool xf = x_fast(x, xdt, k);
@@ -268,7 +268,7 @@ int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stre
             args.count = 0;
         }
         if (ok) {
-            args.p[args.count++] = StreamProblem{(const uint8_t*)p.w, nullptr, p.x, p.y, p.n, p.k, p.fmt, p.fmt,
+            args.p[args.count++] = StreamProblem{(const uint8_t*)p.w, nullptr, p.x, p.y, p.n, p.k, p.fmt, 0,
                                                  p.x_dtype, p.y_dtype, 0, 0};
         }
         if (args.count == STREAM_MAX_PROBLEMS || (!ok && args.count) || (i == count - 1 && args.count)) {

@@ -9,8 +9,7 @@ namespace qmoe {
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ logits, int n, int k,
                                                          float floor_value, int renorm,
                                                          float* __restrict__ weights, int64_t* __restrict__ ids) {
-    extern __shared__ uint32_t keys[];
-    router_row(logits + (size_t)blockIdx.x * n, n, k, floor_value, renorm, keys,
+    router_row(logits + (size_t)blockIdx.x * n, n, k, floor_value, renorm,
                weights + (size_t)blockIdx.x * k, ids + (size_t)blockIdx.x * k);
 }
 
@@ -25,7 +24,7 @@ int router_topk_impl(const float* logits, int tokens, int n, int k, float floor_
     if ((uintptr_t)logits % 4 || (uintptr_t)weights % 4 || (uintptr_t)ids % 8)
         return fail(QMOE_EINVAL, "qmoe_router_topk: misaligned pointer");
     if (tokens == 0) return QMOE_OK;
-    hipLaunchKernelGGL(router_topk_kernel, dim3(tokens), dim3(64), (size_t)n * sizeof(float), s, logits, n, k,
+    hipLaunchKernelGGL(router_topk_kernel, dim3(tokens), dim3(64), 0, s, logits, n, k,
                        floor_value, renorm, weights, ids);
     return check_launch("qmoe_router_topk");
 }

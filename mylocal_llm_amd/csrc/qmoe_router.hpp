@@ -57,47 +57,54 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
 }
 
-// One wave routes one row: full softmax, k rounds of wave-wide arg-best, optional
-// renormalisation.  `keys` (n words) is LDS scratch of the calling wave; n <= 4096 (64 values
-// per lane at most), k <= 32.  Results go to weights[0..k) / ids[0..k) (LDS or global) in
-// selection order; every lane returns with the same view.
-__device__ __forceinline__ void router_row(const float* __restrict__ z, int n, int k, float floor_value, int renorm,
-                                           uint32_t* keys, float* __restrict__ weights, int64_t* __restrict__ ids) {
+// One wave routes one row with the row held in registers (NV values per lane, n <= 64*NV):
+// full softmax, k rounds of wave-wide arg-best, optional renormalisation.  All loads of the
+// row are issued together; nothing in the selection rounds touches memory.  Results go to
+// weights[0..k) / ids[0..k) (LDS or global) in selection order.
+template <int NV>
+__device__ __forceinline__ void router_row_regs(const float* __restrict__ z, int n, int k, float floor_value,
+                                                int renorm, float* __restrict__ weights, int64_t* __restrict__ ids) {
     const int lane = threadIdx.x & 63;
+    float v[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = lane + 64 * j;
+        v[j] = i < n ? z[i] : 0.0f;
+    }
+    unsigned long long cand[NV];
     unsigned long long best = 0ull;
     bool nan_seen = false;
-    for (int i = lane; i < n; i += 64) {
-        const float v = z[i];
-        const uint32_t key = order_key(v);
-        keys[i] = key;
-        nan_seen |= isnan(v);
-        const unsigned long long cand = ((unsigned long long)key << 32) | (uint32_t)~i;
-        best = cand > best ? cand : best;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = lane + 64 * j;
+        const bool valid = i < n;
+        cand[j] = valid ? (((unsigned long long)order_key(v[j]) << 32) | (uint32_t)~i) : 0ull;
+        nan_seen |= valid && isnan(v[j]);
+        best = cand[j] > best ? cand[j] : best;
     }
     const bool any_nan = __any(nan_seen);
     const unsigned long long top = wave_max_u64(best);
     // maximum with NaN propagation, as the portable graph computes it
     const float m = any_nan ? __uint_as_float(0x7FC00000u) : key_value((uint32_t)(top >> 32));
     double part = 0.0;
-    for (int i = lane; i < n; i += 64) part += (double)expf(z[i] - m);
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+        if (lane + 64 * j < n) part += (double)expf(v[j] - m);
     const float denom = (float)wave_sum_f64(part);
-    unsigned long long used = 0ull;  // bit j: this lane's value at index lane + 64*j was taken
     float mass = 0.0f;
-    float mine = 0.0f;               // lane s keeps the probability of selection s
+    float mine = 0.0f;  // lane s keeps the probability of selection s
     long long my_id = 0;
     for (int slot = 0; slot < k; ++slot) {
-        unsigned long long cand = 0ull;
-        for (int i = lane, j = 0; i < n; i += 64, ++j) {
-            const unsigned long long c = ((unsigned long long)keys[i] << 32) | (uint32_t)~i;
-            if (!((used >> j) & 1ull) && c > cand) cand = c;
-        }
-        // a removed or absent entry is 0, below every real candidate (~i is never 0 for i < 2^32-1)
-        const unsigned long long win = wave_max_u64(cand);
-        const int index = (int)~(uint32_t)win;
-        if ((index & 63) == lane) used |= 1ull << (index >> 6);
+        unsigned long long c = 0ull;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) c = cand[j] > c ? cand[j] : c;
+        // a removed or absent entry is 0, below every real candidate (~i is never 0)
+        const unsigned long long win = wave_max_u64(c);
+#pragma unroll
+        for (int j = 0; j < NV; ++j) cand[j] = cand[j] == win ? 0ull : cand[j];  // ids are unique: only the owner matches
         const float p = expf(key_value((uint32_t)(win >> 32)) - m) / denom;
         mass += p;
-        if (lane == slot) { mine = p; my_id = index; }
+        if (lane == slot) { mine = p; my_id = (int)~(uint32_t)win; }
     }
     if (lane < k) {
         float norm = 1.0f;
@@ -105,6 +112,15 @@ __device__ __forceinline__ void router_row(const float* __restrict__ z, int n, i
         weights[lane] = renorm ? mine / norm : mine;
         ids[lane] = my_id;
     }
+}
+
+// One wave routes one row of any supported width (n <= 4096, k <= 32).
+__device__ __forceinline__ void router_row(const float* __restrict__ z, int n, int k, float floor_value, int renorm,
+                                           float* __restrict__ weights, int64_t* __restrict__ ids) {
+    if (n <= 512) router_row_regs<8>(z, n, k, floor_value, renorm, weights, ids);
+    else if (n <= 1024) router_row_regs<16>(z, n, k, floor_value, renorm, weights, ids);
+    else if (n <= 2048) router_row_regs<32>(z, n, k, floor_value, renorm, weights, ids);
+    else router_row_regs<64>(z, n, k, floor_value, renorm, weights, ids);
 }
 
 }  // namespace qmoe

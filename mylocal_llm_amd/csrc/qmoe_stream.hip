@@ -15,10 +15,11 @@ namespace qmoe {
 template <int FMT, bool PAIR>
 __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamArgs args) {
     __shared__ float partial[32 * 2 * 4];
+    __shared__ StreamProblem probs[STREAM_MAX_PROBLEMS];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
-    float xr[64], aux[8];
-    int xgroup = -1, staged = -1;
-    for (int i = 0; i < args.count; ++i) stream_dispatch_shape<FMT, PAIR>(args.p[i], partial, xs, staged, xr, aux, xgroup);
+    if ((int)threadIdx.x < args.count) probs[threadIdx.x] = args.p[threadIdx.x];
+    __syncthreads();
+    stream_run<FMT, PAIR>(probs, args.count, 0, args.flat_items, partial, xs);
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -46,25 +47,30 @@ int stream_grid() {
 // pairs -- as one launch.  All entries must satisfy stream_supported (pairs: both matrices).
 int stream_launch(StreamArgs& args, hipStream_t s) {
     const int grid = stream_grid();
-    const int waves = grid * STREAM_WAVES;
-    long cursor = 0;  // next free worker, counted in waves
+    int flat = 0;   // global work items of the problems whose rows fit one wave
     int group = 0;
     for (int i = 0; i < args.count; ++i) {
         StreamProblem& p = args.p[i];
         const int units = p.k >> 6;
-        const int lr = units <= 8 ? 8 : units <= 16 ? 16 : units <= 32 ? 32 : 64;
-        const int items = (p.n + 64 / lr - 1) / (64 / lr);
         if (units > 64) {  // rows shared by the waves of a workgroup: workgroup-granular round robin
-            p.first_item = (int)((cursor / STREAM_WAVES) % grid);
-            cursor += (long)items * STREAM_WAVES;
+            p.first_item = flat % grid;
+            p.flat_end = 0;
         } else {
-            p.first_item = (int)(cursor % waves);
-            cursor += items;
+            const int rpw = 64 / lanes_per_row(p.k);
+            p.first_item = flat;
+            flat += (p.n + rpw - 1) / rpw;
+            p.flat_end = flat;
         }
         // consecutive problems reading the same activations keep them in registers
         if (i > 0 && (p.x != args.p[i - 1].x || p.k != args.p[i - 1].k || p.xdt != args.p[i - 1].xdt)) ++group;
         p.xgroup = group;
     }
+    // the flat search skips problems with an empty range: give wide problems the running end
+    int running = 0;
+    for (int i = 0; i < args.count; ++i) {
+        if ((args.p[i].k >> 6) > 64) args.p[i].flat_end = running; else running = args.p[i].flat_end;
+    }
+    args.flat_items = flat;
     const dim3 g(grid), b(STREAM_THREADS);
     const bool pair = args.p[0].w2 != nullptr;
 #define QMOE_STREAM(F)                                                                         \

@@ -316,17 +316,24 @@ struct StreamProblem {
     const void* x;      // one activation row
     void* y;            // n outputs
     int n, k;
-    int fmt, fmt2;
+    int fmt;
+    int flat_end;       // rows of up to 4096 columns: end of the problem's range of global work items
     int xdt, ydt;
-    int first_item;     // worker that takes this problem's first row group (round robin across problems)
+    int first_item;     // start of that range; for wider rows the workgroup that takes the first row
     int xgroup;         // equal for consecutive problems that read the same activation row
 };
 
 struct StreamArgs {
     int count;
-    int pad;
+    int flat_items;     // total work items of the problems with rows of up to 4096 columns
     StreamProblem p[STREAM_MAX_PROBLEMS];
 };
+
+// Lanes that share one row of k columns (a power of two, 8..64) and its log2.
+__host__ __device__ inline int lanes_per_row(int k) {
+    const int units = k >> 6;
+    return units <= 8 ? 8 : units <= 16 ? 16 : units <= 32 ? 32 : 64;
+}
 
 // ---- device side of the streaming engine ---------------------------------------------------------
 __device__ __forceinline__ int64_t row_bytes_dev(int fmt, int k) {
@@ -443,18 +450,129 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
     }
 }
 
+// Sum over groups of `lr` consecutive lanes, lr known only at run time (uniform).
+__device__ __forceinline__ float group_sum_rt(float v, int lr) {
+    v = dpp_add<0xB1>(v);
+    v = dpp_add<0x4E>(v);
+    v = dpp_add<0x141>(v);
+    if (lr >= 16) v = dpp_add<0x140>(v);
+    if (lr >= 32) v = dpp_add<0x142, 0xa>(v);
+    if (lr >= 64) v = dpp_add<0x143, 0xc>(v);
+    return v;
+}
+
+// Wave-uniform values moved to scalar registers.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = (uint32_t)uniform((int)(uint32_t)v), hi = (uint32_t)uniform((int)(uint32_t)(v >> 32));
+    return (const uint8_t*)(((uint64_t)hi << 32) | lo);
+}
+
+// All problems whose rows fit one wave (k <= 4096), as ONE stream of work items: item g of the
+// concatenated ranges [first_item, flat_end) belongs to wave g mod W.  A wave requests the
+// rows of its next PD items before it reduces the current one, across problem boundaries, so
+// neither the start of a new matrix nor new activations drain the memory pipeline.
+// Activations are fetched coalesced into the wave's private LDS stripe `xw` and read back as
+// the lane's 64-value slice.  Items [begin, end) are walked; `probs` covers them in order.
+template <int FMT, bool PAIR, int PD>
+__device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, float* xw) {
+    using U = Unit64<FMT>;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int W = gridDim.x * STREAM_WAVES;
+    const int me = blockIdx.x * STREAM_WAVES + wave;
+    int g = begin + ((me - begin % W) + W) % W;
+    if (g >= end) return;
+    RowRegs<FMT, PAIR> buf[PD + 1];
+    int bp[PD + 1], bi[PD + 1];
+    // the problem the fetch side is in, held in scalar registers
+    int cursor = -1, c_begin = 0, c_end = begin, c_n = 1, c_k = 64;
+    const uint8_t *c_w = nullptr, *c_w2 = nullptr;
+    auto fetch = [&](int gi, RowRegs<FMT, PAIR>& r, int& rp, int& ri) {
+        if (gi >= c_end || cursor < 0) {
+            do ++cursor; while (cursor + 1 < count && gi >= uniform(probs[cursor].flat_end));
+            const StreamProblem& p = probs[cursor];
+            c_begin = uniform(p.first_item);
+            c_end = uniform(p.flat_end);
+            c_n = uniform(p.n);
+            c_k = uniform(p.k);
+            c_w = uniform(p.w);
+            if (PAIR) c_w2 = uniform(p.w2);
+        }
+        rp = cursor;
+        ri = gi - c_begin;
+        const int lr = lanes_per_row(c_k), units = c_k >> 6;
+        const int u = lane & (lr - 1);
+        const int uu = u < units ? u : 0;
+        const int row = ri * (64 / lr) + lane / lr;
+        const int64_t rr = row < c_n ? row : (c_n > 0 ? c_n - 1 : 0);
+        const int64_t rb = row_bytes_dev(FMT, c_k);
+        U::load_w(c_w + rr * rb, uu, r.a);
+        if (PAIR) U::load_w(c_w2 + rr * rb, uu, r.b);
+    };
+#pragma unroll
+    for (int j = 0; j < PD; ++j)
+        if (g + j * W < end) fetch(g + j * W, buf[j], bp[j], bi[j]);
+    float xr[64], aux[8];
+    int xgroup = -1;
+    bool done = false;
+    while (!done) {
+#pragma unroll
+        for (int s = 0; s <= PD; ++s) {
+            if (!done) {
+                const int nb = (s + PD) % (PD + 1);
+                if (g + PD * W < end) fetch(g + PD * W, buf[nb], bp[nb], bi[nb]);
+                const StreamProblem& p = probs[bp[s]];
+                const int pk = uniform(p.k), pn = uniform(p.n), pg = uniform(p.xgroup);
+                const int lr = lanes_per_row(pk), units = pk >> 6;
+                const int u = lane & (lr - 1);
+                const bool active = u < units;
+                if (xgroup != pg) {
+                    const uint8_t* px = uniform((const uint8_t*)p.x);
+                    const int pxdt = uniform(p.xdt);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int idx = 4 * lane + 256 * i;
+                        if (idx < pk) *(float4*)(xw + StagedX::at(idx)) = load_x4(px, pxdt, idx);
+                    }
+                    U::load_x(StagedX{xw}, active ? u : 0, xr, aux);
+                    if (!active) {
+#pragma unroll
+                        for (int i = 0; i < 64; ++i) xr[i] = 0.f;
+#pragma unroll
+                        for (int i = 0; i < U::AUX; ++i) aux[i] = 0.f;
+                    }
+                    xgroup = pg;
+                }
+                const int row = bi[s] * (64 / lr) + lane / lr;
+                float v = group_sum_rt(U::dot(buf[s].a, xr, aux), lr);
+                if (PAIR) v = silu_mul(v, group_sum_rt(U::dot(buf[s].b, xr, aux), lr));
+                if (u == lr - 1 && row < pn) store_out(p.y, uniform(p.ydt), row, v);
+                g += W;
+                if (g >= end) done = true;
+            }
+        }
+    }
+}
+
+// Rows requested ahead: bounded by the 256-VGPR budget (a BF16 unit is 32 dwords per row).
+template <int FMT, bool PAIR> struct Prefetch { static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (PAIR ? 1 : 2); };
+
+// A whole problem list held in LDS: first the single stream of all problems whose rows fit a
+// wave, then, one after the other, the problems with wider rows (four waves per row).
 template <int FMT, bool PAIR>
-__device__ __forceinline__ void stream_dispatch_shape(const StreamProblem& p, float* partial, float* xs, int& staged,
-                                                      float (&xr)[64], float (&aux)[8], int& xgroup) {
-    const int units = p.k >> 6;
-    // rows requested ahead: bounded by the 256-VGPR budget (a BF16 unit is 32 dwords per row)
-    constexpr int PD = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (PAIR ? 1 : 2);
-    if (units <= 8) stream_problem<FMT, PAIR, 8, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
-    else if (units <= 16) stream_problem<FMT, PAIR, 16, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
-    else if (units <= 32) stream_problem<FMT, PAIR, 32, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
-    else if (units <= 64) stream_problem<FMT, PAIR, 64, 1, PD>(p, partial, xs, staged, xr, aux, xgroup);
-    else if (units <= 128) stream_problem<FMT, PAIR, 64, 2, PD>(p, partial, xs, staged, xr, aux, xgroup);
-    else stream_problem<FMT, PAIR, 64, 4, PD>(p, partial, xs, staged, xr, aux, xgroup);
+__device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, float* partial, float* xs) {
+    constexpr int PD = Prefetch<FMT, PAIR>::DEPTH;
+    const int wave = threadIdx.x >> 6;
+    if (flat_end > flat_begin) stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES));
+    float xr[64], aux[8];
+    int xgroup = -1, staged = -1;
+    for (int i = 0; i < count; ++i) {
+        const StreamProblem& p = probs[i];
+        if (p.n < 1 || (p.k >> 6) <= 64) continue;
+        if ((p.k >> 6) <= 128) stream_problem<FMT, PAIR, 64, 2, PD>(p, partial, xs, staged, xr, aux, xgroup);
+        else stream_problem<FMT, PAIR, 64, 4, PD>(p, partial, xs, staged, xr, aux, xgroup);
+    }
 }
 
 // True if (fmt, shape, alignment) can go through the streaming kernel.
