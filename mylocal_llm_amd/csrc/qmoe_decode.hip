@@ -18,9 +18,11 @@
 namespace qmoe {
 
 static constexpr int DECODE_MAX_TOKENS = 16;
-static constexpr int LIST_STAGE = 48;  // problem descriptors held in LDS at a time
-// rows of the output one wave produces in the down kernel (a BF16 unit needs twice the registers)
-template <int FMT> struct DownRows { static constexpr int PER_WAVE = FMT == QMOE_FMT_BF16 ? 1 : 2; };
+static constexpr int LIST_STAGE = 96;  // problem descriptors held in LDS at a time
+// rows the down kernel requests ahead of the one it reduces (a BF16 unit needs twice the registers)
+template <int FMT> struct DownDepth { static constexpr int ROWS_AHEAD = FMT == QMOE_FMT_BF16 ? 0 : 2; };
+// the down kernel's LDS row: k*F <= 48*128 routed columns plus up to 2048 shared ones, padded
+static constexpr int DOWN_XS_FLOATS = 8192 + 4 * (8192 / 64);
 
 struct DecodeRouteArgs {
     const float* logits;       // [T, E] or null
@@ -163,7 +165,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
         __syncthreads();
         // the stage's share of the flat item stream (empty when the rows are wider than a wave)
         const int wide = (staged[0].k >> 6) > 64;
-        stream_run<FMT, PAIR>(staged, m, wide ? 0 : staged[0].first_item, wide ? 0 : staged[m - 1].flat_end, partial, xs);
+        stream_run<FMT, PAIR>(staged, m, wide ? 0 : staged[0].first_item, wide ? 0 : staged[m - 1].flat_end, true, partial, xs);
     }
 }
 
@@ -172,11 +174,12 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
 // LDS and no launch sits between the logits and the first expert byte.  Workgroup 0 also
 // publishes the routing for the down kernel.
 static constexpr int FUSED_MAX_TOKENS = 4;
+static constexpr int FUSED_MAX_EXPERTS = 1024;  // wider rows need more registers than the streaming loop leaves
 
 template <int FMT>
 __global__ __launch_bounds__(STREAM_THREADS, 2) void decode_pairs_fused_kernel(const DecodeRouteArgs a) {
     __shared__ float partial[32 * 2 * 4];
-    __shared__ StreamProblem staged[LIST_STAGE];
+    __shared__ StreamProblem staged[FUSED_MAX_TOKENS * 12];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     __shared__ int64_t ids_sel[FUSED_MAX_TOKENS][32];
     __shared__ float w_sel[FUSED_MAX_TOKENS][32];
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void decode_pairs_fused_kernel(c
         const float adm_part = a.shared_gate ? admission_partial(a.hidden, a.xdt, t, a.d, a.shared_gate, lane) : 0.f;
         float adm = adm_part;
         if (a.logits) {
-            router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w_sel[t], ids_sel[t]);
+            router_row<FUSED_MAX_EXPERTS / 64>(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w_sel[t], ids_sel[t]);
         } else if (lane < k) {
             ids_sel[t][lane] = a.in_ids[(size_t)t * k + lane];
             w_sel[t][lane] = a.in_weights[(size_t)t * k + lane];
@@ -261,7 +264,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void decode_pairs_fused_kernel(c
     }
     __syncthreads();
     const int wide = (a.d >> 6) > 64;
-    stream_run<FMT, true>(staged, count, 0, wide ? 0 : staged[count - 1].flat_end, partial, xs);
+    stream_run<FMT, true>(staged, count, 0, wide ? 0 : staged[count - 1].flat_end, a.tokens > 1, partial, xs);
 }
 
 template <int LPE>
@@ -283,15 +286,19 @@ struct DecodeDownArgs {
     const float* sorted_w;      // [T, k]
     const float* sig;           // [T]
     void* out;                  // [T, D]
-    int odt, k, d, f, fsh;
+    int odt, k, d, f, fsh, rows_per_wave;
 };
 
 // Lane layout of a wave: lanes [0, k*LPE) = expert slot j = lane / LPE, part = lane % LPE of
 // the F/128 column parts of its down row; lanes [48, 48 + Fsh/128) = the shared expert's row
-// parts.  Every lane owns two 64-element units (128 columns).
+// parts.  Every lane owns two 64-element units (128 columns) of its expert's h, fetched once
+// per workgroup into padded LDS (coalesced) and kept in registers while the wave walks
+// `rows_per_wave` consecutive output rows with DownDepth rows requested ahead.
 template <int FMT, int LPE>
 __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArgs a) {
     using U = Unit64<FMT>;
+    constexpr int PD = DownDepth<FMT>::ROWS_AHEAD;
+    __shared__ __attribute__((aligned(16))) float xs[DOWN_XS_FLOATS];
     const int t = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int k = a.k;
@@ -306,20 +313,28 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
     const int kk = shared ? a.fsh : a.f;
     const int64_t rbytes = row_bytes_dev(FMT, kk);
     const uint8_t* base = shared ? a.shared_down : a.down + (int64_t)(e >= 0 ? e : 0) * a.down_stride;
-    const float* xsrc = shared ? a.hs + (size_t)t * a.fsh : a.h + ((size_t)t * k + slot) * a.f;
-    constexpr int ROWS = DownRows<FMT>::PER_WAVE;
-    const int row0 = (blockIdx.x * 4 + wave) * ROWS;
-    uint32_t ra[ROWS][2][U::RAW];
+    const int row0 = (blockIdx.x * 4 + wave) * a.rows_per_wave;
+    const int nrows = a.d - row0 < a.rows_per_wave ? a.d - row0 : a.rows_per_wave;
+    uint32_t buf[PD + 1][2][U::RAW];
+    auto fetch = [&](int r, uint32_t (&b)[2][U::RAW]) {
+        const uint8_t* rp = base + (int64_t)(row0 + r) * rbytes;
+        U::load_w(rp, 2 * part, b[0]);
+        U::load_w(rp, 2 * part + 1, b[1]);
+    };
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int row = row0 + r < a.d ? row0 + r : a.d - 1;
-        const uint8_t* rp = base + (int64_t)row * rbytes;
-        U::load_w(rp, 2 * part, ra[r][0]);
-        U::load_w(rp, 2 * part + 1, ra[r][1]);
-    }
+    for (int j = 0; j < PD; ++j)
+        if (j < nrows) fetch(j, buf[j]);
+    // this token's h of every slot, then the shared expert's, as one padded fp32 row in LDS
+    const int nr = k * a.f, total = nr + (a.shared_down ? a.fsh : 0);
+    const float* hr = a.h + (size_t)t * nr;
+    const float* hsh = a.hs + (size_t)t * a.fsh;
+    for (int i = 4 * threadIdx.x; i < total; i += 4 * 256)
+        *(float4*)(xs + StagedX::at(i)) = i < nr ? *(const float4*)(hr + i) : *(const float4*)(hsh + (i - nr));
+    __syncthreads();
+    const int ux = shared ? (nr >> 6) + 2 * part : slot * (a.f >> 6) + 2 * part;
     float x0[64], x1[64], aux0[U::AUX], aux1[U::AUX];
-    U::load_x(GlobalX{xsrc, QMOE_DT_F32}, 2 * part, x0, aux0);
-    U::load_x(GlobalX{xsrc, QMOE_DT_F32}, 2 * part + 1, x1, aux1);
+    U::load_x(StagedX{xs}, ux, x0, aux0);
+    U::load_x(StagedX{xs}, ux + 1, x1, aux1);
     if (!live) {
 #pragma unroll
         for (int i = 0; i < 64; ++i) { x0[i] = 0.f; x1[i] = 0.f; }
@@ -327,23 +342,32 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
         for (int i = 0; i < U::AUX; ++i) { aux0[i] = 0.f; aux1[i] = 0.f; }
     }
     const float sg = a.sig[t];
+    int r = 0;
+    bool done = nrows <= 0;
+    while (!done) {
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        float v = U::dot(ra[r][0], x0, aux0) + U::dot(ra[r][1], x1, aux1);
-        if (!live) v = 0.f;  // idle lanes decoded whatever bytes sit at the base address
-        const float ys = group_sum<16>(v);   // lanes 48..63 are one DPP row: the shared expert's total
-        const float yr = part_sum<LPE>(v);   // every slot's total in each of its lanes
-        float acc = 0.f;
-        for (int j = 0; j < k; ++j) {
-            const float yj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(yr), j * LPE));
-            const float wj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(route_w), j));
-            acc = add_product(acc, yj, wj);
+        for (int s = 0; s <= PD; ++s) {
+            if (!done) {
+                if (r + PD < nrows) fetch(r + PD, buf[(s + PD) % (PD + 1)]);
+                float v = U::dot(buf[s][0], x0, aux0) + U::dot(buf[s][1], x1, aux1);
+                if (!live) v = 0.f;  // idle lanes decoded whatever bytes sit at the base address
+                const float ys = group_sum<16>(v);   // lanes 48..63 are one DPP row: the shared expert's total
+                const float yr = part_sum<LPE>(v);   // every slot's total in each of its lanes
+                float acc = 0.f;
+                for (int j = 0; j < k; ++j) {
+                    const float yj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(yr), j * LPE));
+                    const float wj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(route_w), j));
+                    acc = add_product(acc, yj, wj);
+                }
+                if (a.shared_down) {
+                    const float y63 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ys), 63));
+                    acc = add_product(acc, y63, sg);
+                }
+                if (lane == 0) store_out(a.out, a.odt, (size_t)t * a.d + row0 + r, acc);
+                ++r;
+                if (r >= nrows) done = true;
+            }
         }
-        if (a.shared_down) {
-            const float y63 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ys), 63));
-            acc = add_product(acc, y63, sg);
-        }
-        if (lane == 0 && row0 + r < a.d) store_out(a.out, a.odt, (size_t)t * a.d + row0 + r, acc);
     }
 }
 
@@ -418,7 +442,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     r.tokens = a.tokens;
     r.workers = grid * STREAM_WAVES;
     int rc;
-    const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.tokens * (a.top_k + 1) <= LIST_STAGE;
+    const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.top_k + 1 <= 12 && (!a.logits || b.n_experts <= FUSED_MAX_EXPERTS);
     if (fused) {
         const dim3 fg(grid), fb(STREAM_THREADS);
         switch (b.gate_fmt) {
@@ -457,7 +481,10 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     d.d = b.d_model;
     d.f = b.d_ff;
     d.fsh = r.fsh;
-    const int rows_per_wg = 4 * (b.down_fmt == QMOE_FMT_BF16 ? DownRows<QMOE_FMT_BF16>::PER_WAVE : DownRows<QMOE_FMT_Q8_0>::PER_WAVE);
+    // enough workgroups to fill the chip at one token; longer walks (activations reused) beyond
+    const long want = (long)a.tokens * b.d_model / 2048;
+    d.rows_per_wave = want >= 8 ? 8 : want >= 4 ? 4 : 2;
+    const int rows_per_wg = 4 * d.rows_per_wave;
     const dim3 dgrid((b.d_model + rows_per_wg - 1) / rows_per_wg, a.tokens), dblock(256);
     const int lpe = b.d_ff >> 7;
 #define QMOE_DOWN_L(F, L) hipLaunchKernelGGL((decode_down_kernel<F, L>), dgrid, dblock, 0, s, d)

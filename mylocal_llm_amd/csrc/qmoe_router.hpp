@@ -114,12 +114,14 @@ __device__ __forceinline__ void router_row_regs(const float* __restrict__ z, int
     }
 }
 
-// One wave routes one row of any supported width (n <= 4096, k <= 32).
+// One wave routes one row of any supported width (n <= 64 * MAXNV <= 4096, k <= 32); callers
+// that are short of registers cap the width they accept.
+template <int MAXNV = 64>
 __device__ __forceinline__ void router_row(const float* __restrict__ z, int n, int k, float floor_value, int renorm,
                                            float* __restrict__ weights, int64_t* __restrict__ ids) {
     if (n <= 512) router_row_regs<8>(z, n, k, floor_value, renorm, weights, ids);
-    else if (n <= 1024) router_row_regs<16>(z, n, k, floor_value, renorm, weights, ids);
-    else if (n <= 2048) router_row_regs<32>(z, n, k, floor_value, renorm, weights, ids);
+    else if (n <= 1024 || MAXNV <= 16) router_row_regs<16>(z, n, k, floor_value, renorm, weights, ids);
+    else if (n <= 2048 || MAXNV <= 32) router_row_regs<32>(z, n, k, floor_value, renorm, weights, ids);
     else router_row_regs<64>(z, n, k, floor_value, renorm, weights, ids);
 }
 

@@ -19,7 +19,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamA
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     if ((int)threadIdx.x < args.count) probs[threadIdx.x] = args.p[threadIdx.x];
     __syncthreads();
-    stream_run<FMT, PAIR>(probs, args.count, 0, args.flat_items, partial, xs);
+    stream_run<FMT, PAIR>(probs, args.count, 0, args.flat_items, false, partial, xs);
 }
 
 // ---- host side ---------------------------------------------------------------------------------

@@ -470,18 +470,27 @@ __device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
 }
 
 // All problems whose rows fit one wave (k <= 4096), as ONE stream of work items: item g of the
-// concatenated ranges [first_item, flat_end) belongs to wave g mod W.  A wave requests the
-// rows of its next PD items before it reduces the current one, across problem boundaries, so
-// neither the start of a new matrix nor new activations drain the memory pipeline.
+// concatenated ranges [first_item, flat_end).  Wave w takes items w, w + W, ... (all waves
+// sweep one window of consecutive rows: best for few, long matrices) or, with `contiguous`,
+// one contiguous share (it changes activations as rarely as possible: best for lists of many
+// small matrices over several activation rows).  A wave requests
+// the rows of its next PD items before it reduces the current one, across problem boundaries,
+// so the start of a new matrix does not drain the memory pipeline.
 // Activations are fetched coalesced into the wave's private LDS stripe `xw` and read back as
 // the lane's 64-value slice.  Items [begin, end) are walked; `probs` covers them in order.
 template <int FMT, bool PAIR, int PD>
-__device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, float* xw) {
+__device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, bool contiguous, float* xw) {
     using U = Unit64<FMT>;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = gridDim.x * STREAM_WAVES;
     const int me = blockIdx.x * STREAM_WAVES + wave;
-    int g = begin + ((me - begin % W) + W) % W;
+    int g = begin + me, step = W;
+    if (contiguous) {
+        const int share = (end - begin) / W, extra = (end - begin) % W;
+        g = begin + me * share + (me < extra ? me : extra);
+        end = g + share + (me < extra ? 1 : 0);
+        step = 1;
+    }
     if (g >= end) return;
     RowRegs<FMT, PAIR> buf[PD + 1];
     int bp[PD + 1], bi[PD + 1];
@@ -490,7 +499,15 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
     const uint8_t *c_w = nullptr, *c_w2 = nullptr;
     auto fetch = [&](int gi, RowRegs<FMT, PAIR>& r, int& rp, int& ri) {
         if (gi >= c_end || cursor < 0) {
-            do ++cursor; while (cursor + 1 < count && gi >= uniform(probs[cursor].flat_end));
+            // 64 range ends at a time: one LDS read and a ballot per hop
+            ++cursor;
+            while (true) {
+                const int c = cursor + lane < count ? cursor + lane : count - 1;
+                const uint64_t past = __ballot(gi >= probs[c].flat_end && cursor + lane < count - 1);
+                const int hop = ~past ? __builtin_ctzll(~past) : 64;
+                cursor += hop;
+                if (hop < 64) break;
+            }
             const StreamProblem& p = probs[cursor];
             c_begin = uniform(p.first_item);
             c_end = uniform(p.flat_end);
@@ -512,7 +529,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
     };
 #pragma unroll
     for (int j = 0; j < PD; ++j)
-        if (g + j * W < end) fetch(g + j * W, buf[j], bp[j], bi[j]);
+        if (g + j * step < end) fetch(g + j * step, buf[j], bp[j], bi[j]);
     float xr[64], aux[8];
     int xgroup = -1;
     bool done = false;
@@ -521,7 +538,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
         for (int s = 0; s <= PD; ++s) {
             if (!done) {
                 const int nb = (s + PD) % (PD + 1);
-                if (g + PD * W < end) fetch(g + PD * W, buf[nb], bp[nb], bi[nb]);
+                if (g + PD * step < end) fetch(g + PD * step, buf[nb], bp[nb], bi[nb]);
                 const StreamProblem& p = probs[bp[s]];
                 const int pk = uniform(p.k), pn = uniform(p.n), pg = uniform(p.xgroup);
                 const int lr = lanes_per_row(pk), units = pk >> 6;
@@ -548,7 +565,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
                 float v = group_sum_rt(U::dot(buf[s].a, xr, aux), lr);
                 if (PAIR) v = silu_mul(v, group_sum_rt(U::dot(buf[s].b, xr, aux), lr));
                 if (u == lr - 1 && row < pn) store_out(p.y, uniform(p.ydt), row, v);
-                g += W;
+                g += step;
                 if (g >= end) done = true;
             }
         }
@@ -561,10 +578,10 @@ template <int FMT, bool PAIR> struct Prefetch { static constexpr int DEPTH = FMT
 // A whole problem list held in LDS: first the single stream of all problems whose rows fit a
 // wave, then, one after the other, the problems with wider rows (four waves per row).
 template <int FMT, bool PAIR>
-__device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, float* partial, float* xs) {
+__device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, bool contiguous, float* partial, float* xs) {
     constexpr int PD = Prefetch<FMT, PAIR>::DEPTH;
     const int wave = threadIdx.x >> 6;
-    if (flat_end > flat_begin) stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES));
+    if (flat_end > flat_begin) stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES));
     float xr[64], aux[8];
     int xgroup = -1, staged = -1;
     for (int i = 0; i < count; ++i) {
