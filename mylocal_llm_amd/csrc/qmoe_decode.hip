@@ -47,103 +47,137 @@ struct DecodeRouteArgs {
     int renorm, n_experts, k, d, f, fsh, fmt, xdt, tokens, workers;
 };
 
-// This lane's part of hidden[t] . g; the loads of eight steps travel together.
-__device__ __forceinline__ float admission_partial(const void* hidden, int xdt, int t, int d, const float* g, int lane) {
-    float acc = 0.f;
-    for (int base = 0; base < d; base += 2048) {
-        float4 hv[8], gv[8];
+// hidden[t] . g for the shared expert's admission gate, 2048 columns at a time: issue() only
+// puts the loads in flight, reduce() adds this lane's products to acc.
+struct AdmissionRegs {
+    float4 h[8], g[8];
+    __device__ __forceinline__ void issue(const void* hidden, int xdt, int t, int d, const float* gate, int lane, int base) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int i = base + 4 * lane + 256 * j;
             const bool in = i < d;
-            hv[j] = in ? load_x4(hidden, xdt, t * d + i) : make_float4(0, 0, 0, 0);
-            gv[j] = in ? *(const float4*)(g + i) : make_float4(0, 0, 0, 0);
+            h[j] = in ? load_x4(hidden, xdt, t * d + i) : make_float4(0, 0, 0, 0);
+            g[j] = in ? *(const float4*)(gate + i) : make_float4(0, 0, 0, 0);
         }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc += (hv[j].x * gv[j].x + hv[j].y * gv[j].y) + (hv[j].z * gv[j].z + hv[j].w * gv[j].w);
     }
-    return acc;
+    __device__ __forceinline__ float reduce(float acc) const {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += (h[j].x * g[j].x + h[j].y * g[j].y) + (h[j].z * g[j].z + h[j].w * g[j].w);
+        return acc;
+    }
+};
+
+__device__ __forceinline__ int64_t readlane_i64(int64_t v, int lane) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)v >> 32), lane);
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// One wave routes token t: the row's loads first, then the admission gate's (and whatever
+// `more_loads` issues), then the selection.  The token's selections leave sorted by expert
+// id in sid[0..k) (LDS); with `publish` the wave also writes the routing outputs, the sorted
+// routing and the admission gate for the down kernel.
+template <int MAXNV, typename MoreLoads>
+__device__ __forceinline__ void route_token(const DecodeRouteArgs& a, int t, bool publish, int64_t* sid, MoreLoads&& more_loads) {
+    const int lane = threadIdx.x & 63, k = a.k;
+    AdmissionRegs ar;
+    auto issue = [&] {
+        if (a.shared_gate && publish) ar.issue(a.hidden, a.xdt, t, a.d, a.shared_gate, lane, 0);
+        more_loads();
+    };
+    float w = 0.f;
+    int64_t id = 0;
+    if (a.logits) {
+        router_row<MAXNV>(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w, id, issue);
+    } else {
+        if (lane < k) {
+            id = a.in_ids[(size_t)t * k + lane];
+            w = a.in_weights[(size_t)t * k + lane];
+        }
+        issue();
+    }
+    // rank of this selection in ascending expert id; equal ids keep slot order
+    int rank = 0;
+    for (int j = 0; j < k; ++j) {
+        const int64_t other = readlane_i64(id, j);
+        rank += (other < id) || (other == id && j < lane);
+    }
+    if (lane < k) {
+        sid[rank] = id;
+        if (publish) {
+            const bool ok = id >= 0 && id < a.n_experts;
+            if (!ok) *a.status = 1;
+            if (a.out_weights) {
+                a.out_weights[(size_t)t * k + lane] = w;
+                a.out_ids[(size_t)t * k + lane] = id;
+            }
+            a.sorted_ids[(size_t)t * k + rank] = ok ? (int)id : -1;
+            a.sorted_w[(size_t)t * k + rank] = w;
+        }
+    }
+    if (publish) {
+        float adm = 0.f;
+        if (a.shared_gate) {
+            adm = ar.reduce(adm);
+            for (int base = 2048; base < a.d; base += 2048) {
+                ar.issue(a.hidden, a.xdt, t, a.d, a.shared_gate, lane, base);
+                adm = ar.reduce(adm);
+            }
+            adm = wave_sum(adm);
+        }
+        // sigmoid(hidden . g) without overflow
+        if (lane == 0) a.sig[t] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
+    }
+}
+
+// Entry j of token t's part of the problem list: the gate/up pair of its j-th expert in
+// ascending id (j < k) or of the shared expert (j == k).
+__device__ __forceinline__ StreamProblem decode_problem(const DecodeRouteArgs& a, int t, int j, int64_t e) {
+    const int k = a.k;
+    const int units = a.d >> 6;
+    const int rpw = 64 / lanes_per_row(a.d);
+    const int items_r = (a.f + rpw - 1) / rpw, items_s = a.shared_gate_w ? (a.fsh + rpw - 1) / rpw : 0;
+    const int wide = units > 64 ? STREAM_WAVES : 1;
+    const int64_t xbytes = (int64_t)a.d * (a.xdt == QMOE_DT_F32 ? 4 : 2);
+    const long cursor = ((long)t * ((long)k * items_r + items_s) + (long)j * items_r) * wide;
+    StreamProblem p;
+    p.x = (const uint8_t*)a.hidden + (size_t)t * xbytes;
+    p.k = a.d;
+    p.fmt = a.fmt;
+    p.xdt = a.xdt;
+    p.ydt = QMOE_DT_F32;
+    p.xgroup = t;
+    if (j < k) {
+        const bool ok = e >= 0 && e < a.n_experts;
+        const int64_t ee = ok ? e : 0;
+        p.w = a.gate + ee * a.gate_stride;
+        p.w2 = a.up + ee * a.up_stride;
+        p.y = a.h + ((size_t)t * k + j) * a.f;
+        p.n = ok ? a.f : 0;  // an out-of-range id contributes nothing (its h stays unused)
+    } else {
+        p.w = a.shared_gate_w;
+        p.w2 = a.shared_up_w;
+        p.y = a.hs + (size_t)t * a.fsh;
+        p.n = a.fsh;
+    }
+    if (units > 64) {
+        p.first_item = (int)((cursor / STREAM_WAVES) % (a.workers / STREAM_WAVES));
+        p.flat_end = 0;
+    } else {
+        p.first_item = (int)cursor;
+        p.flat_end = (int)cursor + (j < k ? items_r : items_s);
+    }
+    return p;
 }
 
 __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs a) {
-    __shared__ int64_t ids_sel[32];
-    __shared__ float w_sel[32];
-    __shared__ int order[32];
+    __shared__ int64_t sid[32];
     const int t = blockIdx.x, lane = threadIdx.x;
-    const int k = a.k;
-    // admission gate first: its loads are in flight while the row is routed
-    float adm = a.shared_gate ? admission_partial(a.hidden, a.xdt, t, a.d, a.shared_gate, lane) : 0.f;
-    if (a.logits) {
-        router_row(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w_sel, ids_sel);
-    } else if (lane < k) {
-        ids_sel[lane] = a.in_ids[(size_t)t * k + lane];
-        w_sel[lane] = a.in_weights[(size_t)t * k + lane];
-    }
+    route_token<64>(a, t, true, sid, [] {});
     __syncthreads();
-    if (lane < k) {
-        if (a.out_weights) {
-            a.out_weights[(size_t)t * k + lane] = w_sel[lane];
-            a.out_ids[(size_t)t * k + lane] = ids_sel[lane];
-        }
-        // rank of this selection in ascending expert id; equal ids keep slot order
-        const int64_t mine = ids_sel[lane];
-        int rank = 0;
-        for (int j = 0; j < k; ++j) rank += (ids_sel[j] < mine) || (ids_sel[j] == mine && j < lane);
-        order[rank] = lane;
-    }
-    __syncthreads();
-    if (a.shared_gate) adm = wave_sum(adm);
-    if (lane == 0) {
-        // sigmoid(hidden . g) without overflow
-        a.sig[t] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
-        if (t == 0) *a.problem_count = a.tokens * (k + (a.shared_gate_w ? 1 : 0));
-    }
-    // this token's problems, in sorted-slot order, then the shared expert
-    const int units = a.d >> 6;
-    const int lr = units <= 8 ? 8 : units <= 16 ? 16 : units <= 32 ? 32 : 64;
-    const int rpw = 64 / lr;
-    const int items_r = (a.f + rpw - 1) / rpw, items_s = a.shared_gate_w ? (a.fsh + rpw - 1) / rpw : 0;
-    const int per_token = k + (a.shared_gate_w ? 1 : 0);
-    const int64_t xbytes = (int64_t)a.d * (a.xdt == QMOE_DT_F32 ? 4 : 2);
-    const long token_cursor = (long)t * ((long)k * items_r + items_s) * (units > 64 ? STREAM_WAVES : 1);
-    if (lane <= k && lane < per_token) {
-        StreamProblem p;
-        p.x = (const uint8_t*)a.hidden + (size_t)t * xbytes;
-        p.k = a.d;
-        p.fmt = a.fmt;
-        p.xdt = a.xdt;
-        p.ydt = QMOE_DT_F32;
-        p.xgroup = t;
-        long cursor;
-        if (lane < k) {
-            const int s = order[lane];
-            const int64_t e = ids_sel[s];
-            const bool ok = e >= 0 && e < a.n_experts;
-            if (!ok) *a.status = 1;
-            const int64_t ee = ok ? e : 0;
-            p.w = a.gate + ee * a.gate_stride;
-            p.w2 = a.up + ee * a.up_stride;
-            p.y = a.h + ((size_t)t * k + lane) * a.f;
-            p.n = ok ? a.f : 0;  // an out-of-range id contributes nothing (its h stays unused)
-            a.sorted_ids[(size_t)t * k + lane] = ok ? (int)e : -1;
-            a.sorted_w[(size_t)t * k + lane] = w_sel[s];
-            cursor = token_cursor + (long)lane * items_r * (units > 64 ? STREAM_WAVES : 1);
-        } else {
-            p.w = a.shared_gate_w;
-            p.w2 = a.shared_up_w;
-            p.y = a.hs + (size_t)t * a.fsh;
-            p.n = a.fsh;
-            cursor = token_cursor + (long)k * items_r * (units > 64 ? STREAM_WAVES : 1);
-        }
-        if (units > 64) {
-            p.first_item = (int)((cursor / STREAM_WAVES) % (a.workers / STREAM_WAVES));
-            p.flat_end = 0;
-        } else {
-            p.first_item = (int)cursor;
-            p.flat_end = (int)cursor + (lane < k ? items_r : items_s);
-        }
-        a.problems[(size_t)t * per_token + lane] = p;
-    }
+    const int per_token = a.k + (a.shared_gate_w ? 1 : 0);
+    if (lane == 0 && t == 0) *a.problem_count = a.tokens * per_token;
+    if (lane < per_token) a.problems[(size_t)t * per_token + lane] = decode_problem(a, t, lane, lane < a.k ? sid[lane] : 0);
 }
 
 // The streaming engine over a problem list that lives in device memory.
@@ -169,102 +203,53 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
     }
 }
 
-// Routing fused into the gate/up launch (up to FUSED_MAX_TOKENS tokens): every workgroup
-// routes the tokens itself (its four waves share them), so the problem list never leaves
-// LDS and no launch sits between the logits and the first expert byte.  Workgroup 0 also
-// publishes the routing for the down kernel.
+// Routing fused into the gate/up launch (up to FUSED_MAX_TOKENS tokens of up to 4096
+// columns): every workgroup routes the tokens itself (one wave per token), so the problem
+// list never leaves LDS and no launch sits between the logits and the first expert byte.
+// While the routing loads travel, the workgroup also fetches the tokens' activations into
+// LDS, stripe t for token t, where the streaming loop picks them up.  Workgroup 0 publishes
+// the routing for the down kernel.
 static constexpr int FUSED_MAX_TOKENS = 4;
 static constexpr int FUSED_MAX_EXPERTS = 1024;  // wider rows need more registers than the streaming loop leaves
+static constexpr int FUSED_MAX_SLOTS = 12;      // top_k + shared expert
 
 template <int FMT>
 __global__ __launch_bounds__(STREAM_THREADS, 2) void decode_pairs_fused_kernel(const DecodeRouteArgs a) {
-    __shared__ float partial[32 * 2 * 4];
-    __shared__ StreamProblem staged[FUSED_MAX_TOKENS * 12];
+    __shared__ StreamProblem staged[FUSED_MAX_TOKENS * FUSED_MAX_SLOTS];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
-    __shared__ int64_t ids_sel[FUSED_MAX_TOKENS][32];
-    __shared__ float w_sel[FUSED_MAX_TOKENS][32];
-    __shared__ int order[FUSED_MAX_TOKENS][32];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ int64_t sid[FUSED_MAX_TOKENS][32];
+    constexpr int STRIPE = STREAM_XS_FLOATS / STREAM_WAVES;
+    const int wave = threadIdx.x >> 6;
     const int k = a.k, tokens = a.tokens;
-    for (int t = wave; t < tokens; t += STREAM_WAVES) {
-        const float adm_part = a.shared_gate ? admission_partial(a.hidden, a.xdt, t, a.d, a.shared_gate, lane) : 0.f;
-        float adm = adm_part;
-        if (a.logits) {
-            router_row<FUSED_MAX_EXPERTS / 64>(a.logits + (size_t)t * a.n_experts, a.n_experts, k, a.floor_value, a.renorm, w_sel[t], ids_sel[t]);
-        } else if (lane < k) {
-            ids_sel[t][lane] = a.in_ids[(size_t)t * k + lane];
-            w_sel[t][lane] = a.in_weights[(size_t)t * k + lane];
+    // this thread's share of the tokens' activations: columns 4*tid + 1024*i of every token
+    float4 xv[FUSED_MAX_TOKENS][4];
+    auto fetch_x = [&] {
+#pragma unroll
+        for (int t = 0; t < FUSED_MAX_TOKENS; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = 4 * threadIdx.x + 1024 * i;
+                if (t < tokens && col < a.d) xv[t][i] = load_x4(a.hidden, a.xdt, t * a.d + col);
+            }
+    };
+    if (wave < tokens) route_token<FUSED_MAX_EXPERTS / 64>(a, wave, blockIdx.x == 0, sid[wave], fetch_x);
+    else fetch_x();
+#pragma unroll
+    for (int t = 0; t < FUSED_MAX_TOKENS; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int col = 4 * threadIdx.x + 1024 * i;
+            if (t < tokens && col < a.d) *(float4*)(xs + t * STRIPE + StagedX::at(col)) = xv[t][i];
         }
-        if (a.shared_gate) adm = wave_sum(adm);
-        if (blockIdx.x == 0 && lane == 0)
-            a.sig[t] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
-    }
-    __syncthreads();
-    if ((int)threadIdx.x < tokens * k) {
-        const int t = threadIdx.x / k, s = threadIdx.x % k;
-        const int64_t mine = ids_sel[t][s];
-        int rank = 0;
-        for (int j = 0; j < k; ++j) rank += (ids_sel[t][j] < mine) || (ids_sel[t][j] == mine && j < s);
-        order[t][rank] = s;
-        if (blockIdx.x == 0 && a.out_weights) {
-            a.out_weights[(size_t)t * k + s] = w_sel[t][s];
-            a.out_ids[(size_t)t * k + s] = mine;
-        }
-    }
     __syncthreads();
     const int per_token = k + (a.shared_gate_w ? 1 : 0);
     const int count = tokens * per_token;
     if ((int)threadIdx.x < count) {
         const int t = threadIdx.x / per_token, j = threadIdx.x % per_token;
-        const int units = a.d >> 6;
-        const int lr = units <= 8 ? 8 : units <= 16 ? 16 : units <= 32 ? 32 : 64;
-        const int rpw = 64 / lr;
-        const int items_r = (a.f + rpw - 1) / rpw, items_s = a.shared_gate_w ? (a.fsh + rpw - 1) / rpw : 0;
-        const int wide = units > 64 ? STREAM_WAVES : 1;
-        const int64_t xbytes = (int64_t)a.d * (a.xdt == QMOE_DT_F32 ? 4 : 2);
-        const long token_cursor = (long)t * ((long)k * items_r + items_s) * wide;
-        StreamProblem p;
-        p.x = (const uint8_t*)a.hidden + (size_t)t * xbytes;
-        p.k = a.d;
-        p.fmt = a.fmt;
-        p.xdt = a.xdt;
-        p.ydt = QMOE_DT_F32;
-        p.xgroup = t;
-        long cursor;
-        if (j < k) {
-            const int s = order[t][j];
-            const int64_t e = ids_sel[t][s];
-            const bool ok = e >= 0 && e < a.n_experts;
-            const int64_t ee = ok ? e : 0;
-            p.w = a.gate + ee * a.gate_stride;
-            p.w2 = a.up + ee * a.up_stride;
-            p.y = a.h + ((size_t)t * k + j) * a.f;
-            p.n = ok ? a.f : 0;
-            if (blockIdx.x == 0) {
-                if (!ok) *a.status = 1;
-                a.sorted_ids[(size_t)t * k + j] = ok ? (int)e : -1;
-                a.sorted_w[(size_t)t * k + j] = w_sel[t][s];
-            }
-            cursor = token_cursor + (long)j * items_r * wide;
-        } else {
-            p.w = a.shared_gate_w;
-            p.w2 = a.shared_up_w;
-            p.y = a.hs + (size_t)t * a.fsh;
-            p.n = a.fsh;
-            cursor = token_cursor + (long)k * items_r * wide;
-        }
-        if (units > 64) {
-            p.first_item = (int)((cursor / STREAM_WAVES) % (a.workers / STREAM_WAVES));
-            p.flat_end = 0;
-        } else {
-            p.first_item = (int)cursor;
-            p.flat_end = (int)cursor + (j < k ? items_r : items_s);
-        }
-        staged[threadIdx.x] = p;
+        staged[threadIdx.x] = decode_problem(a, t, j, j < k ? sid[t][j] : 0);
     }
     __syncthreads();
-    const int wide = (a.d >> 6) > 64;
-    stream_run<FMT, true>(staged, count, 0, wide ? 0 : staged[count - 1].flat_end, a.tokens > 1, partial, xs);
+    stream_run<FMT, true, false>(staged, count, 0, staged[count - 1].flat_end, tokens > 1, nullptr, xs, xs);
 }
 
 template <int LPE>
@@ -442,7 +427,8 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     r.tokens = a.tokens;
     r.workers = grid * STREAM_WAVES;
     int rc;
-    const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.top_k + 1 <= 12 && (!a.logits || b.n_experts <= FUSED_MAX_EXPERTS);
+    const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.top_k + 1 <= FUSED_MAX_SLOTS && b.d_model <= 4096 &&
+                       (!a.logits || b.n_experts <= FUSED_MAX_EXPERTS);
     if (fused) {
         const dim3 fg(grid), fb(STREAM_THREADS);
         switch (b.gate_fmt) {

@@ -1,5 +1,5 @@
 // Router: full softmax over all experts, exact top-k selection, optional renormalisation
-// of the selected mass.  One wave per token row; the row lives in LDS, selection is k
+// of the selected mass.  One wave per token row; the row lives in registers, selection is k
 // rounds of a wave-wide arg-best under the reference's order (descending value, NaN last,
 // lower id on ties: mini_llm/ops/router_decode.py:19-26).
 #include "qmoe_router.hpp"
@@ -9,8 +9,13 @@ namespace qmoe {
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ logits, int n, int k,
                                                          float floor_value, int renorm,
                                                          float* __restrict__ weights, int64_t* __restrict__ ids) {
-    router_row(logits + (size_t)blockIdx.x * n, n, k, floor_value, renorm,
-               weights + (size_t)blockIdx.x * k, ids + (size_t)blockIdx.x * k);
+    float w;
+    int64_t id;
+    router_row(logits + (size_t)blockIdx.x * n, n, k, floor_value, renorm, w, id, [] {});
+    if ((int)threadIdx.x < k) {
+        weights[(size_t)blockIdx.x * k + threadIdx.x] = w;
+        ids[(size_t)blockIdx.x * k + threadIdx.x] = id;
+    }
 }
 
 int router_topk_impl(const float* logits, int tokens, int n, int k, float floor_value, int renorm, float* weights,

@@ -477,9 +477,11 @@ __device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
 // the rows of its next PD items before it reduces the current one, across problem boundaries,
 // so the start of a new matrix does not drain the memory pipeline.
 // Activations are fetched coalesced into the wave's private LDS stripe `xw` and read back as
-// the lane's 64-value slice.  Items [begin, end) are walked; `probs` covers them in order.
+// the lane's 64-value slice; with `xpre` the caller has already put the activations of
+// xgroup g into stripe g of that array (same padded layout) and nothing is fetched here.  Items [begin, end) are walked; `probs` covers them in order.
 template <int FMT, bool PAIR, int PD>
-__device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, bool contiguous, float* xw) {
+__device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, bool contiguous, float* xw,
+                                            const float* xpre) {
     using U = Unit64<FMT>;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = gridDim.x * STREAM_WAVES;
@@ -545,14 +547,19 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
                 const int u = lane & (lr - 1);
                 const bool active = u < units;
                 if (xgroup != pg) {
-                    const uint8_t* px = uniform((const uint8_t*)p.x);
-                    const int pxdt = uniform(p.xdt);
+                    const float* xl = xw;
+                    if (xpre) {
+                        xl = xpre + pg * (STREAM_XS_FLOATS / STREAM_WAVES);
+                    } else {
+                        const uint8_t* px = uniform((const uint8_t*)p.x);
+                        const int pxdt = uniform(p.xdt);
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int idx = 4 * lane + 256 * i;
-                        if (idx < pk) *(float4*)(xw + StagedX::at(idx)) = load_x4(px, pxdt, idx);
+                        for (int i = 0; i < 16; ++i) {
+                            const int idx = 4 * lane + 256 * i;
+                            if (idx < pk) *(float4*)(xw + StagedX::at(idx)) = load_x4(px, pxdt, idx);
+                        }
                     }
-                    U::load_x(StagedX{xw}, active ? u : 0, xr, aux);
+                    U::load_x(StagedX{xl}, active ? u : 0, xr, aux);
                     if (!active) {
 #pragma unroll
                         for (int i = 0; i < 64; ++i) xr[i] = 0.f;
@@ -577,11 +584,14 @@ template <int FMT, bool PAIR> struct Prefetch { static constexpr int DEPTH = FMT
 
 // A whole problem list held in LDS: first the single stream of all problems whose rows fit a
 // wave, then, one after the other, the problems with wider rows (four waves per row).
-template <int FMT, bool PAIR>
-__device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, bool contiguous, float* partial, float* xs) {
+template <int FMT, bool PAIR, bool WIDE = true>
+__device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, bool contiguous, float* partial, float* xs,
+                                           const float* xpre = nullptr) {
     constexpr int PD = Prefetch<FMT, PAIR>::DEPTH;
     const int wave = threadIdx.x >> 6;
-    if (flat_end > flat_begin) stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES));
+    if (flat_end > flat_begin)
+        stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES), xpre);
+    if (!WIDE) return;
     float xr[64], aux[8];
     int xgroup = -1, staged = -1;
     for (int i = 0; i < count; ++i) {
