@@ -9,6 +9,7 @@
 //   pos_of[T*k]       sorted position of assignment (t, slot)
 //   hidden_act[A, F]  fp32 SwiGLU activations, terms[A, D] fp32 weighted expert outputs
 // with A = T*k.  Nothing is read back by the host.
+#include "qmoe_gemm.hpp"
 #include "qmoe_rowdot.hpp"
 #include "qmoe_stream.hpp"
 
@@ -21,6 +22,7 @@ int router_topk_impl(const float* logits, int tokens, int n, int k, float floor_
                      int64_t* ids, hipStream_t s);
 
 static constexpr int PLAN_THREADS = 1024;
+static constexpr int GEMM_MIN_TOKENS = 17;  // fewer tokens take the decode path
 static constexpr size_t PLAN_LDS_LIMIT = 60 * 1024;
 
 // Block-wide exclusive scan of one int per thread (PLAN_THREADS threads); returns the
@@ -55,7 +57,11 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
                                                                  int* __restrict__ active, int* __restrict__ n_active,
                                                                  int* __restrict__ sorted_token,
                                                                  float* __restrict__ sorted_weight,
-                                                                 int* __restrict__ pos_of, int* __restrict__ status) {
+                                                                 int* __restrict__ pos_of, int* __restrict__ status,
+                                                                 int* __restrict__ chunk_expert,
+                                                                 int* __restrict__ chunk_start,
+                                                                 int* __restrict__ chunk_count,
+                                                                 int* __restrict__ n_chunks) {
     extern __shared__ uint32_t selection[];  // n_experts*words bitmap, then n_experts offsets
     __shared__ int wave_sums[PLAN_THREADS / 64];
     __shared__ int total;
@@ -77,25 +83,35 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
     // Per-thread chunk of consecutive experts -> counts -> two scans (sizes, non-empty flags).
     const int chunk = (n_experts + PLAN_THREADS - 1) / PLAN_THREADS;
     const int first = tid * chunk;
-    int my_count = 0, my_active = 0;
+    int my_count = 0, my_active = 0, my_chunks = 0;
     for (int e = first; e < first + chunk && e < n_experts; ++e) {
         int c = 0;
         for (int w = 0; w < words; ++w) c += __popc(selection[e * words + w]);
         my_count += c;
         my_active += c > 0;
+        my_chunks += (c + GEMM_CHUNK - 1) / GEMM_CHUNK;
     }
     int count_prefix = block_exclusive_scan(my_count, wave_sums, &total);
     const int all = total;
     int active_prefix = block_exclusive_scan(my_active, wave_sums, &total);
+    const int all_active = total;
+    int chunk_prefix = block_exclusive_scan(my_chunks, wave_sums, &total);
     for (int e = first; e < first + chunk && e < n_experts; ++e) {
         int c = 0;
         for (int w = 0; w < words; ++w) c += __popc(selection[e * words + w]);
         offsets[e] = count_prefix;
         expert_offset[e] = count_prefix;
+        // the expert's assignments in chunks of GEMM_CHUNK tokens, for the token-tile GEMM
+        for (int at = 0; at < c; at += GEMM_CHUNK) {
+            chunk_expert[chunk_prefix] = e;
+            chunk_start[chunk_prefix] = count_prefix + at;
+            chunk_count[chunk_prefix] = c - at < GEMM_CHUNK ? c - at : GEMM_CHUNK;
+            ++chunk_prefix;
+        }
         count_prefix += c;
         if (c > 0) active[active_prefix++] = e;
     }
-    if (tid == 0) { offsets[n_experts] = all; *n_active = total; }
+    if (tid == 0) { offsets[n_experts] = all; *n_active = all_active; *n_chunks = total; }
     __syncthreads();
     for (int a = tid; a < assignments; a += PLAN_THREADS) {
         const int64_t e64 = ids[a];
@@ -293,7 +309,8 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MoeWorkspace {
     size_t weights, ids, offsets, active, n_active, status, sorted_token, sorted_weight, pos_of, hidden_act, terms,
-        shared_h, shared_out, sig, problems, total;
+        shared_h, shared_out, sig, problems, chunk_expert, chunk_start, chunk_count, n_chunks, total;
+    int max_chunks;
 };
 
 static MoeWorkspace moe_layout(int tokens, int k, int n_experts, int d_model, int d_ff, int d_ff_shared) {
@@ -316,6 +333,12 @@ static MoeWorkspace moe_layout(int tokens, int k, int n_experts, int d_model, in
     w.shared_out = take((size_t)tokens * d_model * 4);
     w.sig = take((size_t)tokens * 4);
     w.problems = take(a * 64 + (size_t)tokens * 64);  // device-side problem list of the decode path
+    // every expert with assignments ends in one partly filled chunk at most
+    w.max_chunks = (int)(a / GEMM_CHUNK + (a < (size_t)n_experts ? a : (size_t)n_experts));
+    w.chunk_expert = take((size_t)w.max_chunks * 4);
+    w.chunk_start = take((size_t)w.max_chunks * 4);
+    w.chunk_count = take((size_t)w.max_chunks * 4);
+    w.n_chunks = take(4);
     w.total = at;
     return w;
 }
@@ -339,6 +362,98 @@ static void launch_gate_up(const qmoe_moe_args& a, const MoeWorkspace& L, char* 
     else if (a.tokens <= 16) QMOE_GU(4);
     else QMOE_GU(8);
 #undef QMOE_GU
+}
+
+// ---- token batches on MFMA ----------------------------------------------------------------------
+// SwiGLU activations travel between the two GEMMs as bf16 hi / lo arrays; they take the place
+// of the fp32 activations in the workspace (2 x 2 bytes per element).
+static bool gemm_path(const qmoe_moe_args& a, const char* ws, const MoeWorkspace& L) {
+    const qmoe_expert_bank& b = a.bank;
+    if (a.tokens < GEMM_MIN_TOKENS) return false;
+    if (b.gate_fmt != b.up_fmt) return false;
+    if (!gemm_supported(b.gate_fmt, b.gate, b.gate_stride, b.d_ff, b.d_model, a.hidden, a.hidden_dtype, b.d_model)) return false;
+    if (!gemm_supported(b.up_fmt, b.up, b.up_stride, b.d_ff, b.d_model, a.hidden, a.hidden_dtype, b.d_model)) return false;
+    if (!gemm_supported(b.down_fmt, b.down, b.down_stride, b.d_model, b.d_ff, ws + L.hidden_act, GEMM_A_PAIR, b.d_ff)) return false;
+    if ((size_t)a.tokens * a.top_k * b.d_ff * 2 % 16) return false;  // the lo array starts 16-byte aligned
+    if (a.shared_gate_w) {
+        if (a.shared_gate_fmt != a.shared_up_fmt) return false;
+        if (!gemm_supported(a.shared_gate_fmt, a.shared_gate_w, 0, a.d_ff_shared, b.d_model, a.hidden, a.hidden_dtype, b.d_model)) return false;
+        if (!gemm_supported(a.shared_up_fmt, a.shared_up_w, 0, a.d_ff_shared, b.d_model, a.hidden, a.hidden_dtype, b.d_model)) return false;
+        if (!gemm_supported(a.shared_down_fmt, a.shared_down_w, 0, b.d_model, a.d_ff_shared, ws + L.shared_h, GEMM_A_PAIR, a.d_ff_shared)) return false;
+        if ((size_t)a.tokens * a.d_ff_shared * 2 % 16) return false;
+    }
+    return true;
+}
+
+static int launch_combine(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L, const float* shared_out, hipStream_t s);
+
+// After the plan: grouped gate/up + SwiGLU, grouped down * route, the shared expert, combine.
+static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L, hipStream_t s) {
+    const qmoe_expert_bank& b = a.bank;
+    const size_t assignments = (size_t)a.tokens * a.top_k;
+    int rc;
+    GemmArgs g{};
+    g.w = (const uint8_t*)b.gate;
+    g.w2 = (const uint8_t*)b.up;
+    g.stride = b.gate_stride;
+    g.stride2 = b.up_stride;
+    g.n = b.d_ff;
+    g.k = b.d_model;
+    g.a0 = a.hidden;
+    g.a_stride = b.d_model;
+    g.gather = (const int*)(ws + L.sorted_token);
+    g.chunk_expert = (const int*)(ws + L.chunk_expert);
+    g.chunk_start = (const int*)(ws + L.chunk_start);
+    g.chunk_count = (const int*)(ws + L.chunk_count);
+    g.n_chunks = (const int*)(ws + L.n_chunks);
+    uint16_t* h_hi = (uint16_t*)(ws + L.hidden_act);
+    uint16_t* h_lo = h_hi + assignments * b.d_ff;
+    g.out0 = h_hi;
+    g.out1 = h_lo;
+    if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, s))) return rc;
+    GemmArgs d = g;
+    d.w = (const uint8_t*)b.down;
+    d.w2 = nullptr;
+    d.stride = b.down_stride;
+    d.n = b.d_model;
+    d.k = b.d_ff;
+    d.a0 = h_hi;
+    d.a1 = h_lo;
+    d.a_stride = b.d_ff;
+    d.gather = nullptr;
+    d.out0 = ws + L.terms;
+    d.out1 = nullptr;
+    d.scale = (const float*)(ws + L.sorted_weight);
+    if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, s))) return rc;
+    const float* shared_out = nullptr;
+    if (a.shared_gate_w) {
+        const int chunks = (a.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
+        GemmArgs sg{};
+        sg.w = (const uint8_t*)a.shared_gate_w;
+        sg.w2 = (const uint8_t*)a.shared_up_w;
+        sg.n = a.d_ff_shared;
+        sg.k = b.d_model;
+        sg.a0 = a.hidden;
+        sg.a_stride = b.d_model;
+        sg.dense_tokens = a.tokens;
+        uint16_t* s_hi = (uint16_t*)(ws + L.shared_h);
+        uint16_t* s_lo = s_hi + (size_t)a.tokens * a.d_ff_shared;
+        sg.out0 = s_hi;
+        sg.out1 = s_lo;
+        if ((rc = gemm_launch(a.shared_gate_fmt, true, a.hidden_dtype, sg, chunks, s))) return rc;
+        GemmArgs sd{};
+        sd.w = (const uint8_t*)a.shared_down_w;
+        sd.n = b.d_model;
+        sd.k = a.d_ff_shared;
+        sd.a0 = s_hi;
+        sd.a1 = s_lo;
+        sd.a_stride = a.d_ff_shared;
+        sd.dense_tokens = a.tokens;
+        sd.out0 = ws + L.shared_out;
+        if ((rc = gemm_launch(a.shared_down_fmt, false, GEMM_A_PAIR, sd, chunks, s))) return rc;
+        shared_out = (const float*)(ws + L.shared_out);
+    }
+    return launch_combine(a, ws, L, shared_out, s);
 }
 
 int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_bytes, hipStream_t s) {
@@ -397,10 +512,12 @@ int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_b
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, s, ids, weights, a.tokens, a.top_k,
                        b.n_experts, (int*)(ws + L.offsets), (int*)(ws + L.active), (int*)(ws + L.n_active),
                        (int*)(ws + L.sorted_token), (float*)(ws + L.sorted_weight), (int*)(ws + L.pos_of),
-                       (int*)(ws + L.status));
+                       (int*)(ws + L.status), (int*)(ws + L.chunk_expert), (int*)(ws + L.chunk_start),
+                       (int*)(ws + L.chunk_count), (int*)(ws + L.n_chunks));
     if ((rc = check_launch("qmoe_moe_forward(plan)"))) return rc;
     const int assignments = a.tokens * a.top_k;
     const int max_active = assignments < b.n_experts ? assignments : b.n_experts;
+    if (gemm_path(a, ws, L)) return gemm_forward(a, ws, L, s);
     const bool xf = x_fast(a.hidden, a.hidden_dtype, b.d_model);
     if (a.hidden_dtype == QMOE_DT_F32) launch_gate_up<QMOE_DT_F32>(a, L, ws, max_active, xf, s);
     else if (a.hidden_dtype == QMOE_DT_F16) launch_gate_up<QMOE_DT_F16>(a, L, ws, max_active, xf, s);
@@ -431,6 +548,11 @@ int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_b
         if (rc) return rc;
         shared_out = (const float*)(ws + L.shared_out);
     }
+    return launch_combine(a, ws, L, shared_out, s);
+}
+
+static int launch_combine(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L, const float* shared_out, hipStream_t s) {
+    const qmoe_expert_bank& b = a.bank;
     const dim3 cgrid(a.tokens), cblock(256);
 #define QMOE_COMBINE(XDT)                                                                                            \
     hipLaunchKernelGGL((moe_combine_kernel<XDT>), cgrid, cblock, 0, s, (const float*)(ws + L.terms),                 \

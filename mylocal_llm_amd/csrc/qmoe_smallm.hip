@@ -7,41 +7,14 @@
 // fp32 / fp16 activations are split the same way, bf16 activations are used as they are.
 // hi*hi + lo*hi + hi*lo accumulate in the MFMA's fp32 accumulator.  A workgroup owns a tile
 // of 16*RT rows; its four waves take every fourth group of units and meet in LDS at the end.
+#include "qmoe_mfma.hpp"
 #include "qmoe_rowdot.hpp"
 #include "qmoe_stream.hpp"
 
 namespace qmoe {
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-
 static constexpr int SM_THREADS = 256;
 static constexpr int SM_WAVES = 4;
-
-// bf16 pair from two floats that are exactly representable (upper halves of the fp32 words)
-__device__ __forceinline__ uint32_t pack_exact_bf16(float a, float b) {
-    return (__float_as_uint(a) >> 16) | (__float_as_uint(b) & 0xFFFF0000u);
-}
-
-union OperandBits {
-    bf16x8 v;
-    uint32_t u[4];
-};
-
-// Eight fp32 values -> two bf16 terms: hi = the value rounded to nearest bf16, lo = the exact
-// remainder rounded to nearest bf16; hi + lo carries 16 significant bits of each value.
-__device__ __forceinline__ void split_terms(const float* v, OperandBits& hi, OperandBits& lo) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float a = v[2 * i], b = v[2 * i + 1];
-        hi.v[2 * i] = (__bf16)a;
-        hi.v[2 * i + 1] = (__bf16)b;
-        const float ra = a - __uint_as_float(hi.u[i] << 16);
-        const float rb = b - __uint_as_float(hi.u[i] & 0xFFFF0000u);
-        lo.v[2 * i] = (__bf16)ra;
-        lo.v[2 * i + 1] = (__bf16)rb;
-    }
-}
 
 // The eight activation values k0..k0+7 of one token as MFMA A operands: one bf16 term for
 // bf16 input, else hi + lo (rounded remainder): 16 significant bits.
@@ -66,7 +39,6 @@ __device__ __forceinline__ void load_a_terms(const void* x, size_t index, bool v
 }
 
 template <int XDT> struct ATerms { static constexpr int N = XDT == QMOE_DT_BF16 ? 1 : 2; };
-template <int FMT> struct BTerms { static constexpr int N = FMT == QMOE_FMT_BF16 ? 1 : 2; };
 
 // MT token tiles of 16, RT row tiles of 16 per workgroup item.  Lane (n = l%16, g = l/16) of
 // wave w owns unit 16*step + 4*w + g of row n: it loads the unit with the streaming engine's

@@ -300,3 +300,38 @@ def test_prefill_config_512_tokens_zipf(cuda):
     want, _, want_ids = oracle_step(hidden[picks[:2]], logits[picks[:2]], k, gate, up, down, shared, gate_vec)
     np.testing.assert_array_equal(ids.cpu().numpy()[picks[:2]], want_ids)
     assert rel_l2(out.cpu().numpy()[picks[:2]], want) <= 2e-5
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "BF16"])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_moe_token_batches_ragged_shapes(cuda, fmt, dtype):
+    """Token batches beyond the decode sizes with a width that is not a multiple of 256 columns
+    (a partly filled last pass), row counts that are not multiples of the row tiles, experts with
+    0, 1, 17 and more than 32 tokens, and fp16 / fp32 hidden states."""
+    announce("moe token batches ragged", fmt, dtype)
+    e, d, f, fsh, k, t = 8, 320, 192, 128, 3, 77
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh, (fmt, fmt, fmt), 1300)
+    hidden = synthetic.activations((t, d), 11) * np.float32(2.0)
+    if dtype == "f16":
+        hidden = hidden.astype(np.float16).astype(np.float32)
+    logits = synthetic.router_logits(t, e, 13)
+    logits[:, 5] = -30.0            # an expert nobody selects
+    logits[1:, 6] = -30.0           # an expert with exactly one token
+    logits[0, 6] = 30.0
+    logits[:17, 7] = 20.0           # ... with 17 tokens
+    logits[17:, 7] = -30.0
+    logits[:, 2] += 10.0            # ... with all 77 tokens: three chunks
+    assert not synthetic.has_topk_ties(logits, k)
+    want, want_w, want_ids = oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec)
+    counts = np.bincount(want_ids.ravel(), minlength=e)
+    assert counts[5] == 0 and counts[6] == 1 and counts[7] == 17 and counts[2] == t
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    dshared = tuple(upload(w, cuda) for w in shared)
+    hd = torch.from_numpy(hidden).to(cuda)
+    if dtype == "f16":
+        hd = hd.half()
+    out, w, ids = moe_step(hd, bank, k, logits=torch.from_numpy(logits).to(cuda), shared=dshared,
+                           shared_gate=torch.from_numpy(gate_vec).to(cuda), return_routing=True)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    tol = 2e-5 if dtype == "f32" else 1e-3  # fp16 output rounding
+    assert rel_l2(out.float().cpu().numpy(), want) <= tol <= REL_L2
