@@ -18,8 +18,32 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamA
     __shared__ StreamProblem probs[STREAM_MAX_PROBLEMS];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     if ((int)threadIdx.x < args.count) probs[threadIdx.x] = args.p[threadIdx.x];
+    // every activation row the flat stream will need, fetched together: a wave that moves on to
+    // the next matrix finds its activations in LDS instead of waiting for them
+    if (args.groups > 0) {
+        constexpr int STRIPE = STREAM_XS_FLOATS / STREAM_WAVES;
+        float4 v[STREAM_WAVES][4];
+#pragma unroll
+        for (int g = 0; g < STREAM_WAVES; ++g) {
+            const StreamProblem& p = args.p[args.group_problem[g < args.groups ? g : 0]];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = 4 * threadIdx.x + 1024 * i;
+                if (g < args.groups && col < p.k) v[g][i] = load_x4(p.x, p.xdt, col);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < STREAM_WAVES; ++g) {
+            const int pk = args.p[args.group_problem[g < args.groups ? g : 0]].k;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = 4 * threadIdx.x + 1024 * i;
+                if (g < args.groups && col < pk) *(float4*)(xs + g * STRIPE + StagedX::at(col)) = v[g][i];
+            }
+        }
+    }
     __syncthreads();
-    stream_run<FMT, PAIR>(probs, args.count, 0, args.flat_items, false, partial, xs);
+    stream_run<FMT, PAIR>(probs, args.count, 0, args.flat_items, false, partial, xs, args.groups > 0 ? xs : nullptr);
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -48,7 +72,9 @@ int stream_grid() {
 int stream_launch(StreamArgs& args, hipStream_t s) {
     const int grid = stream_grid();
     int flat = 0;   // global work items of the problems whose rows fit one wave
-    int group = 0;
+    int group = -1, wide_group = 1 << 20;
+    const StreamProblem *last_narrow = nullptr, *last_wide = nullptr;
+    bool fits = true;
     for (int i = 0; i < args.count; ++i) {
         StreamProblem& p = args.p[i];
         const int units = p.k >> 6;
@@ -61,10 +87,23 @@ int stream_launch(StreamArgs& args, hipStream_t s) {
             flat += (p.n + rpw - 1) / rpw;
             p.flat_end = flat;
         }
-        // consecutive problems reading the same activations keep them in registers
-        if (i > 0 && (p.x != args.p[i - 1].x || p.k != args.p[i - 1].k || p.xdt != args.p[i - 1].xdt)) ++group;
-        p.xgroup = group;
+        // consecutive problems reading the same activations keep them in registers; the groups
+        // of the flat stream are numbered 0, 1, ... (their LDS stripes), the others apart
+        if (units > 64) {
+            if (last_wide && (p.x != last_wide->x || p.k != last_wide->k || p.xdt != last_wide->xdt)) ++wide_group;
+            p.xgroup = wide_group;
+            last_wide = &p;
+        } else {
+            if (!last_narrow || p.x != last_narrow->x || p.k != last_narrow->k || p.xdt != last_narrow->xdt) {
+                ++group;
+                if (group < STREAM_WAVES) args.group_problem[group] = i; else fits = false;
+            }
+            p.xgroup = group;
+            last_narrow = &p;
+        }
     }
+    args.groups = fits ? group + 1 : 0;
+    for (int g = args.groups > 0 ? args.groups : 0; g < STREAM_WAVES; ++g) args.group_problem[g] = 0;
     // the flat search skips problems with an empty range: give wide problems the running end
     int running = 0;
     for (int i = 0; i < args.count; ++i) {

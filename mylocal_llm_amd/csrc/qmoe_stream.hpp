@@ -326,6 +326,11 @@ struct StreamProblem {
 struct StreamArgs {
     int count;
     int flat_items;     // total work items of the problems with rows of up to 4096 columns
+    // Activation rows of the problems with rows of up to 4096 columns, when there are at most
+    // STREAM_WAVES different ones: group g is read by problem group_problem[g] (and others) and
+    // is fetched into LDS stripe g before the first row is multiplied.
+    int groups;
+    int group_problem[STREAM_WAVES];
     StreamProblem p[STREAM_MAX_PROBLEMS];
 };
 
@@ -580,7 +585,9 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
 }
 
 // Rows requested ahead: bounded by the 256-VGPR budget (a BF16 unit is 32 dwords per row).
-template <int FMT, bool PAIR> struct Prefetch { static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (PAIR ? 1 : 2); };
+template <int FMT, bool PAIR> struct Prefetch {
+    static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (FMT == QMOE_FMT_Q8_0 ? (PAIR ? 1 : 2) : (PAIR ? 1 : 4));
+};
 
 // A whole problem list held in LDS: first the single stream of all problems whose rows fit a
 // wave, then, one after the other, the problems with wider rows (four waves per row).
