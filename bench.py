@@ -215,6 +215,70 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup):
             "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
 
 
+def moe_prefill_extra(torch, lib, device, fmt, tokens, steps, warmup):
+    """512-expert top-10 MoE step at prefill size: Zipf(1.1) expert popularity over a seeded
+    permutation, routing from logits, token-tile MFMA GEMMs, fp32 output [T, 2048]."""
+    import numpy as np
+    from mylocal_llm_amd import _lib, synthetic
+    from mylocal_llm_amd.moe import DevicePackedExpertBank
+    from mylocal_llm_amd.quantized_linear import DevicePackedGGUFWeight
+    e, d, f, fsh, k = 512, 2048, 512, 2048, 10
+    gen = torch.Generator(device=device)
+    gen.manual_seed(11)
+    n_banks = 2
+    banks, shareds = [], []
+    for _ in range(n_banks):
+        g = device_blocks(torch, fmt, e * f, d, gen, device)
+        u = device_blocks(torch, fmt, e * f, d, gen, device)
+        dn = device_blocks(torch, fmt, e * d, f, gen, device)
+        banks.append(DevicePackedExpertBank((g, (e, f, d), fmt), (u, (e, f, d), fmt), (dn, (e, d, f), fmt)))
+        shareds.append(tuple(DevicePackedGGUFWeight(device_blocks(torch, fmt, n, kk, gen, device), (n, kk), fmt)
+                             for n, kk in ((fsh, d), (fsh, d), (d, fsh))))
+    hidden = torch.randn((tokens, d), device=device, generator=gen).to(torch.bfloat16)
+    logits_np = np.stack([synthetic.router_logits(tokens, e, 9 + i, zipf=1.1) for i in range(n_banks)])
+    logits = torch.from_numpy(logits_np).to(device)
+    gate_vec = torch.randn(d, device=device, generator=gen) * 0.02
+    out = torch.empty((tokens, d), device=device, dtype=torch.float32)
+    nbytes_ws = lib.qmoe_moe_workspace_bytes(tokens, k, e, d, f, fsh)
+    workspace = torch.empty(nbytes_ws, dtype=torch.uint8, device=device)
+    calls = []
+    for i in range(n_banks):
+        a = _lib.MoeArgs()
+        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), 2, tokens, k
+        a.logits, a.floor_value, a.renormalize = logits[i].data_ptr(), 2.0 ** -14, 1
+        banks[i].fill(a.bank)
+        g, u, dn = shareds[i]
+        a.shared_gate_w, a.shared_up_w, a.shared_down_w = g.data.data_ptr(), u.data.data_ptr(), dn.data.data_ptr()
+        a.shared_gate_fmt = a.shared_up_fmt = a.shared_down_fmt = _lib.FORMAT_ID[fmt]
+        a.d_ff_shared, a.shared_gate = fsh, gate_vec.data_ptr()
+        a.out, a.out_dtype = out.data_ptr(), 0
+        calls.append(a)
+    state = {"i": 0}
+    wsp = ctypes.c_void_p(workspace.data_ptr())
+
+    def fn(stream):
+        a = calls[state["i"] % n_banks]
+        state["i"] += 1
+        rc = lib.qmoe_moe_forward(ctypes.byref(a), wsp, nbytes_ws, stream)
+        if rc:
+            raise RuntimeError(lib.qmoe_last_error().decode())
+
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    ids = np.argsort(-logits_np, axis=-1, kind="stable")[..., :k]
+    counts = [np.bincount(ids[i].ravel(), minlength=e) for i in range(n_banks)]
+    distinct = float(np.mean([(c > 0).sum() for c in counts]))
+    # tokens are multiplied in tiles of 16 per expert: the MFMA work actually issued
+    padded = float(np.mean([(np.ceil(c / 16) * 16).sum() for c in counts]))
+    nbytes = distinct * 3 * weight_bytes(fmt, f, d) + 3 * weight_bytes(fmt, fsh, d)
+    flops = 2.0 * (tokens * k) * 3 * f * d + 2.0 * tokens * 3 * fsh * d
+    per_step = ms / steps * 1e-3
+    return {"workload": f"moe_prefill_{fmt}_T{tokens}_zipf1.1", "ms_per_step": round(ms / steps, 4),
+            "weight_bytes": int(nbytes), "distinct_experts": distinct, "max_tokens_per_expert": int(max(c.max() for c in counts)),
+            "GBps": round(nbytes / per_step / 1e9, 1), "frac_hbm_peak": round(nbytes / per_step / 1e9 / HBM_PEAK_GBS, 4),
+            "useful_TFLOPs": round(flops / per_step / 1e12, 2), "padded_assignments": padded,
+            "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -223,6 +287,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode"], default=None,
+                    help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device tensor copy (a kernel of known traffic, "
                          "used to scale FETCH_SIZE / WRITE_SIZE counters)")
@@ -240,6 +306,12 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.only == "moe_prefill":
+        print(json.dumps(moe_prefill_extra(torch, lib, device, "Q8_0", 512, max(4, args.steps), args.warmup)))
+        return
+    if args.only == "moe_decode":
+        print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup) for t in (1, 4, 16)]))
+        return
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
@@ -292,6 +364,8 @@ def main():
         for fmt, tokens in (("Q8_0", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q6_K", 1)):
             extras.append(moe_decode_extra(torch, lib, device, fmt, tokens, max(8, args.steps), 3))
             torch.cuda.empty_cache()
+        extras.append(moe_prefill_extra(torch, lib, device, "Q8_0", 512, 6, 2))
+        torch.cuda.empty_cache()
         result["extras"] = extras
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()

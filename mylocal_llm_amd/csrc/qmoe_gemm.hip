@@ -138,6 +138,14 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
 #pragma unroll
             for (int j = 0; j < NS; ++j) stage_load<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
         }
+        // a unit past the end of the row multiplies as zeros: all-zero bytes decode to 0.0 in
+        // every format (zero scales)
+        if (!live) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < U::RAW; ++i) raw[j][i] = 0u;
+        }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -152,12 +160,6 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
                     else {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) bt[0].u[i] = pack_exact_bf16(wf[8 * s + 2 * i], wf[8 * s + 2 * i + 1]);
-                    }
-                    if (!live) {
-#pragma unroll
-                        for (int tb = 0; tb < NB; ++tb)
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) bt[tb].u[i] = 0u;
                     }
                 }
                 const int koff = (U::kstep(uu, s) - 256 * p) * 2;
