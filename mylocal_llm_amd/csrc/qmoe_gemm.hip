@@ -48,14 +48,14 @@ __device__ __forceinline__ void stage_load(uint4& r0, uint4& r1, const GemmArgs&
     if (!valid) { r0 = zero; r1 = zero; }
 }
 
-// ... and their bf16 terms into the staged tile (hi at `dst`, lo one term further).
-template <int AKIND>
+// ... and their bf16 terms into the staged tile (hi at `dst`, lo TERM bytes further).
+template <int AKIND, int TERM>
 __device__ __forceinline__ void stage_store(const uint4 r0, const uint4 r1, uint8_t* dst) {
     if (AKIND == GEMM_A_BF16) {
         *(uint4*)dst = r0;
     } else if (AKIND == GEMM_A_PAIR) {
         *(uint4*)dst = r0;
-        *(uint4*)(dst + GEMM_TERM_BYTES) = r1;
+        *(uint4*)(dst + TERM) = r1;
     } else {
         float v[8];
         if (AKIND == GEMM_A_F32) {
@@ -70,65 +70,83 @@ __device__ __forceinline__ void stage_store(const uint4 r0, const uint4 r1, uint
         OperandBits hi, lo;
         split_terms(v, hi, lo);
         *(uint4*)dst = make_uint4(hi.u[0], hi.u[1], hi.u[2], hi.u[3]);
-        *(uint4*)(dst + GEMM_TERM_BYTES) = make_uint4(lo.u[0], lo.u[1], lo.u[2], lo.u[3]);
+        *(uint4*)(dst + TERM) = make_uint4(lo.u[0], lo.u[1], lo.u[2], lo.u[3]);
     }
 }
 
 // One chunk (expert e, sorted positions start .. start+count) x this workgroup's rows.
-template <int FMT, int AKIND, bool PAIR, int MT>
-__device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, uint8_t* lds) {
+// NM matrices per wave: the gate and up rows of the same index (PAIR, NM == 2) or NM tiles of
+// 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows.
+// With SOLO (one token tile, long rows) the four waves share the same 16 * NM rows and split K:
+// wave w walks its quarter of the passes, stages its own activations in its own part of the
+// LDS tile without waiting for the others, and the partial sums meet in LDS at the end.  A
+// matrix with few rows and many columns then has four times as many, four times shorter,
+// work items.
+template <int FMT, int AKIND, bool PAIR, int NM, int MT, bool SOLO>
+__device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds) {
+    static_assert(!PAIR || NM == 2, "a pair is two matrices");
+    static_assert(!SOLO || (MT == 1 && !PAIR), "a wave stages one token tile on its own");
     using U = Unit64<FMT>;
     constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2, NB = BTerms<FMT>::N;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 15, g = lane >> 4;
-    const int units = a.k >> 6, passes = (units + 3) >> 2;
+    const int units = a.k >> 6, all_passes = (units + 3) >> 2;
+    const int share = SOLO ? (all_passes + 3) >> 2 : all_passes;
+    const int p_begin = SOLO ? wave * share : 0;
+    const int passes = p_begin + share < all_passes ? p_begin + share : all_passes;  // end of this wave's range
     const int64_t rb = row_bytes_dev(FMT, a.k);
-    // two matrices per wave: gate and up rows of the same index, or two 16-row tiles
-    int rows[2];
-    const uint8_t* rp[2];
+    int rows[NM];
+    const uint8_t* rp[NM];
     if (PAIR) {
-        rows[0] = rows[1] = blockIdx.x * 64 + wave * 16 + col;
+        rows[0] = rows[NM - 1] = rowblock * 64 + wave * 16 + col;
         const int64_t rr = rows[0] < a.n ? rows[0] : a.n - 1;
         rp[0] = a.w + (int64_t)e * a.stride + rr * rb;
-        rp[1] = a.w2 + (int64_t)e * a.stride2 + rr * rb;
+        rp[NM - 1] = a.w2 + (int64_t)e * a.stride2 + rr * rb;
     } else {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            rows[j] = blockIdx.x * 128 + wave * 32 + 16 * j + col;
+        for (int j = 0; j < NM; ++j) {
+            rows[j] = SOLO ? rowblock * (16 * NM) + 16 * j + col : rowblock * (64 * NM) + wave * (16 * NM) + 16 * j + col;
             const int64_t rr = rows[j] < a.n ? rows[j] : a.n - 1;
             rp[j] = a.w + (int64_t)e * a.stride + rr * rb;
         }
     }
-    floatx4 acc[2][MT];
+    floatx4 acc[NM][MT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NM; ++j)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    // staging share of this thread: column chunk c8 of token rows tid/32 + 8*j
-    constexpr int NS = 2 * MT;
+    // staging share of this thread: column chunk c8 of token rows tid/32 + 8*j (of the wave's
+    // own copy: rows lane/32 + 2*j)
+    constexpr int NS = SOLO ? 8 : 2 * MT;
+    constexpr int RSTEP = SOLO ? 2 : 8;
     const int c8 = tid & 31;
+    const int r0 = SOLO ? (lane >> 5) : (tid >> 5);
+    if (SOLO) lds += wave * ((AKIND == GEMM_A_BF16 ? 1 : 2) * 16 * GEMM_A_STRIDE);
+    constexpr int TERM = SOLO ? 16 * GEMM_A_STRIDE : GEMM_TERM_BYTES;
     int64_t arow[NS];
     bool avalid[NS];
 #pragma unroll
     for (int j = 0; j < NS; ++j) {
-        const int r = (tid >> 5) + 8 * j;
+        const int r = r0 + RSTEP * j;
         avalid[j] = r < count;
         arow[j] = avalid[j] ? (a.gather ? a.gather[start + r] : start + r) : 0;
     }
     uint4 st0[NS], st1[NS];
-    uint32_t raw[2][U::RAW];
+    uint32_t raw[NM][U::RAW];
     {
-        const int u = g < units ? g : 0;
+        const int u = 4 * p_begin + g < units ? 4 * p_begin + g : 0;
+        const int c0 = 256 * p_begin + 8 * c8;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) U::load_w(rp[j], u, raw[j]);
+        for (int j = 0; j < NM; ++j) U::load_w(rp[j], u, raw[j]);
 #pragma unroll
-        for (int j = 0; j < NS; ++j) stage_load<AKIND>(st0[j], st1[j], a, arow[j], 8 * c8, avalid[j] && 8 * c8 < a.k);
+        for (int j = 0; j < NS; ++j) stage_load<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
     }
-    for (int p = 0; p < passes; ++p) {
-        __syncthreads();  // the previous pass has been multiplied
+    for (int p = p_begin; p < passes; ++p) {
+        // the previous pass has been multiplied (LDS operations of one wave stay in order)
+        if (SOLO) __builtin_amdgcn_wave_barrier(); else __syncthreads();
 #pragma unroll
-        for (int j = 0; j < NS; ++j) stage_store<AKIND>(st0[j], st1[j], lds + ((tid >> 5) + 8 * j) * GEMM_A_STRIDE + 16 * c8);
-        __syncthreads();
+        for (int j = 0; j < NS; ++j) stage_store<AKIND, TERM>(st0[j], st1[j], lds + (r0 + RSTEP * j) * GEMM_A_STRIDE + 16 * c8);
+        if (SOLO) __builtin_amdgcn_wave_barrier(); else __syncthreads();
         const int unit = 4 * p + g;
         const bool live = unit < units;
         const int uu = live ? unit : 0;
@@ -142,12 +160,12 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
         // every format (zero scales)
         if (!live) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < NM; ++j)
 #pragma unroll
                 for (int i = 0; i < U::RAW; ++i) raw[j][i] = 0u;
         }
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < NM; ++j) {
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
                 // the eight weights of step s only: the rest of the unit's decode is dead code
@@ -172,7 +190,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
                     floatx4 c = acc[j][mt];
                     c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, bt[0].v, c, 0, 0, 0);
                     if (NA == 2) {
-                        const uint4 t1 = *(const uint4*)(ap + GEMM_TERM_BYTES);
+                        const uint4 t1 = *(const uint4*)(ap + TERM);
                         a1.u[0] = t1.x; a1.u[1] = t1.y; a1.u[2] = t1.z; a1.u[3] = t1.w;
                         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1.v, bt[0].v, c, 0, 0, 0);
                     }
@@ -182,6 +200,22 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
             }
             // this matrix's unit of the next pass takes the registers that just became free
             if (p + 1 < passes) U::load_w(rp[j], un, raw[j]);
+        }
+    }
+    if (SOLO) {
+        // partial sums of the four K ranges: every wave leaves its own in its own LDS part
+        floatx4* mine = (floatx4*)lds;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < NM; ++j) mine[j * 64 + lane] = acc[j][0];
+        __syncthreads();
+        if (wave != 0) return;
+        constexpr int PART = (AKIND == GEMM_A_BF16 ? 1 : 2) * 16 * GEMM_A_STRIDE / (int)sizeof(floatx4);
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            const floatx4 b = mine[PART + j * 64 + lane], c = mine[2 * PART + j * 64 + lane], d = mine[3 * PART + j * 64 + lane];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][0][i] = (acc[j][0][i] + b[i]) + (c[i] + d[i]);
         }
     }
     // lane (col, g) holds outputs of tokens 16*mt + 4*g + i, row index col of each matrix
@@ -195,7 +229,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
             if (PAIR) {
                 if (rows[0] < a.n) {
                     // SwiGLU, left as two bf16 terms for the down step's A operand
-                    const float v = silu_mul(acc[0][mt][i], acc[1][mt][i]);
+                    const float v = silu_mul(acc[0][mt][i], acc[NM - 1][mt][i]);
                     const uint16_t hi = float_to_bf16_bits(v);
                     const uint16_t lo = float_to_bf16_bits(v - __uint_as_float((uint32_t)hi << 16));
                     ((uint16_t*)a.out0)[pos * a.n + rows[0]] = hi;
@@ -203,11 +237,12 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
+                for (int j = 0; j < NM; ++j) {
                     if (rows[j] >= a.n) continue;
                     const float v = acc[j][mt][i];
                     // the routed product is rounded on its own, as the reference stores it
-                    ((float*)a.out0)[pos * a.n + rows[j]] = a.scale ? mul_unfused(v, a.scale[pos]) : v;
+                    if (a.scale) ((float*)a.out0)[pos * a.n + rows[j]] = mul_unfused(v, a.scale[pos]);
+                    else store_out(a.out0, a.out_dt, pos * a.n + rows[j], v);
                 }
             }
         }
@@ -229,8 +264,35 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_kernel(const GemmAr
         count = a.dense_tokens - start < GEMM_CHUNK ? a.dense_tokens - start : GEMM_CHUNK;
     }
     if (count <= 0) return;
-    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, 1>(a, e, start, count, lds);
-    else tile_gemm_chunk<FMT, AKIND, PAIR, 2>(a, e, start, count, lds);
+    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, 2, 1, false>(a, e, start, count, blockIdx.x, lds);
+    else tile_gemm_chunk<FMT, AKIND, PAIR, 2, 2, false>(a, e, start, count, blockIdx.x, lds);
+}
+
+// Several dense matrices (y = W x for `tokens` rows of x each) in one launch: blockIdx.x walks
+// the row blocks of all problems, blockIdx.y the token chunks.
+template <int FMT, int AKIND, int NM>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_dense_kernel(const GemmDenseArgs d) {
+    constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * NA * GEMM_TERM_BYTES];  // four solo tiles or one shared tile
+    int i = 0;
+    while (i + 1 < d.count && (int)blockIdx.x >= d.block_start[i + 1]) ++i;
+    const bool ksplit = d.p[i].ksplit != 0;
+    const int chunk = ksplit ? 16 : GEMM_CHUNK;
+    const int start = blockIdx.y * chunk;
+    const int count = d.tokens - start < chunk ? d.tokens - start : chunk;
+    if (count <= 0) return;
+    GemmArgs a{};
+    a.w = d.p[i].w;
+    a.n = d.p[i].n;
+    a.k = d.p[i].k;
+    a.a0 = d.p[i].x;
+    a.a_stride = d.p[i].k;
+    a.out0 = d.p[i].y;
+    a.out_dt = d.p[i].ydt;
+    const int rowblock = blockIdx.x - d.block_start[i];
+    if (ksplit) tile_gemm_chunk<FMT, AKIND, false, NM, 1, true>(a, 0, start, count, rowblock, lds);
+    else if (count <= 16) tile_gemm_chunk<FMT, AKIND, false, NM, 1, false>(a, 0, start, count, rowblock, lds);
+    else tile_gemm_chunk<FMT, AKIND, false, NM, 2, false>(a, 0, start, count, rowblock, lds);
 }
 
 // ---- host side ------------------------------------------------------------------------------------
@@ -267,6 +329,50 @@ int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, h
     }
 #undef QMOE_GEMM_F
     return check_launch("token-tile GEMM");
+}
+
+template <int FMT, int NM>
+static void gemm_dense_f(const GemmDenseArgs& d, int a_kind, dim3 grid, hipStream_t s) {
+    const dim3 block(GEMM_THREADS);
+    switch (a_kind) {
+    case GEMM_A_F32: hipLaunchKernelGGL((tile_gemm_dense_kernel<FMT, GEMM_A_F32, NM>), grid, block, 0, s, d); break;
+    case GEMM_A_F16: hipLaunchKernelGGL((tile_gemm_dense_kernel<FMT, GEMM_A_F16, NM>), grid, block, 0, s, d); break;
+    default: hipLaunchKernelGGL((tile_gemm_dense_kernel<FMT, GEMM_A_BF16, NM>), grid, block, 0, s, d); break;
+    }
+}
+
+int stream_grid();
+
+// Row blocks of 128 rows when that still fills the chip, else of 64.
+int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
+    const int chunks = (d.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
+    int blocks128 = 0;
+    for (int i = 0; i < d.count; ++i) blocks128 += (d.p[i].n + 127) / 128;
+    // two row tiles per wave only where the registers hold them without spilling
+    const bool roomy = fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_BF16;
+    const int nm = roomy && blocks128 * chunks >= stream_grid() ? 2 : 1;
+    // rows of 8192 columns and more are shared by the four waves (K split), 16 tokens a chunk
+    int at = 0, ychunks = chunks;
+    for (int i = 0; i < d.count; ++i) {
+        d.p[i].ksplit = d.p[i].k >= 8192;
+        const int rows_per_block = d.p[i].ksplit ? 16 * nm : 64 * nm;
+        d.block_start[i] = at;
+        at += (d.p[i].n + rows_per_block - 1) / rows_per_block;
+        if (d.p[i].ksplit && (d.tokens + 15) / 16 > ychunks) ychunks = (d.tokens + 15) / 16;
+    }
+    d.block_start[d.count] = at;
+    const dim3 grid(at, ychunks);
+#define QMOE_DENSE_F(F)                                        \
+    if (nm == 2) gemm_dense_f<F, 2>(d, a_kind, grid, s);      \
+    else gemm_dense_f<F, 1>(d, a_kind, grid, s)
+    switch (fmt) {
+    case QMOE_FMT_Q8_0: QMOE_DENSE_F(QMOE_FMT_Q8_0); break;
+    case QMOE_FMT_Q6_K: QMOE_DENSE_F(QMOE_FMT_Q6_K); break;
+    case QMOE_FMT_Q5_K: QMOE_DENSE_F(QMOE_FMT_Q5_K); break;
+    default: QMOE_DENSE_F(QMOE_FMT_BF16); break;
+    }
+#undef QMOE_DENSE_F
+    return check_launch("token-tile GEMM (dense)");
 }
 
 }  // namespace qmoe

@@ -29,10 +29,29 @@ struct GemmArgs {
     void* out0;
     void* out1;
     const float* scale;
+    int out_dt;              // element type of an unscaled plain output
+};
+
+static constexpr int GEMM_MAX_PROBLEMS = 16;
+
+// Dense matrices sharing the packed format, the activation element type and the token count.
+struct GemmDenseProblem {
+    const uint8_t* w;
+    const void* x;           // [tokens, k]
+    void* y;                 // [tokens, n]
+    int n, k, ydt;
+    int ksplit;              // set by the launcher: the four waves of a workgroup split K
+};
+struct GemmDenseArgs {
+    int count, tokens;
+    int block_start[GEMM_MAX_PROBLEMS + 1];
+    GemmDenseProblem p[GEMM_MAX_PROBLEMS];
 };
 
 bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const void* a0, int a_kind, int64_t a_stride);
 // grid = (row blocks, chunks); `chunks` is an upper bound when the list lives on the device
 int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, hipStream_t s);
+// fills block_start and launches
+int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s);
 
 }  // namespace qmoe

@@ -7,6 +7,7 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include "qmoe_gemm.hpp"
 #include "qmoe_rowdot.hpp"
 #include "qmoe_stream.hpp"
 
@@ -137,7 +138,19 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
         args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, 0, xdt, ydt, 0, 0};
         return stream_launch(args, s);
     }
-    if (smallm_supported(fmt, w, n, k, x, xdt, tokens)) return smallm_launch(fmt, w, n, k, x, xdt, tokens, y, ydt, s);
+    // token batches: the token-tile GEMM when its 64-row blocks fill the chip (or the batch is
+    // beyond the small-batch kernel), else the small-batch kernel with its 16-row tiles
+    const bool tile_ok = tokens >= 2 && gemm_supported(fmt, w, 0, n, k, x, xdt, k);
+    const bool small_ok = smallm_supported(fmt, w, n, k, x, xdt, tokens);
+    const long tile_groups = (long)((n + 63) / 64) * ((tokens + GEMM_CHUNK - 1) / GEMM_CHUNK);
+    if (tile_ok && (!small_ok || tile_groups >= stream_grid() / 2)) {
+        GemmDenseArgs d{};
+        d.count = 1;
+        d.tokens = tokens;
+        d.p[0] = GemmDenseProblem{(const uint8_t*)w, x, y, n, k, ydt, 0};
+        return gemm_dense_launch(fmt, xdt, d, s);
+    }
+    if (small_ok) return smallm_launch(fmt, w, n, k, x, xdt, tokens, y, ydt, s);
     const bool fast = rows_fast(fmt, w, row_bytes(fmt, k), k) && x_fast(x, xdt, k);
     if (xdt == QMOE_DT_F32) launch_linear_mt<QMOE_DT_F32>(w, fmt, n, k, fast, x, tokens, y, ydt, s);
     else if (xdt == QMOE_DT_F16) launch_linear_mt<QMOE_DT_F16>(w, fmt, n, k, fast, x, tokens, y, ydt, s);
@@ -256,31 +269,49 @@ int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stre
             return fail(QMOE_EINVAL, "qmoe_linear_batch: problem %d has a null pointer, no tokens or a bad element type", i);
     }
     // Single-token problems the streaming kernel covers share launches (up to
-    // STREAM_MAX_PROBLEMS each); anything else goes through the general kernels in order.
+    // STREAM_MAX_PROBLEMS each), and so do token batches of one size the token-tile GEMM covers
+    // (up to GEMM_MAX_PROBLEMS each); anything else goes through linear_impl in order.
     StreamArgs args{};
+    GemmDenseArgs dense{};
+    int dense_fmt = 0, dense_xdt = 0;
+    auto flush_stream = [&]() -> int {
+        if (!args.count) return QMOE_OK;
+        const int rc = stream_launch(args, (hipStream_t)stream);
+        args.count = 0;
+        return rc;
+    };
+    auto flush_dense = [&]() -> int {
+        if (!dense.count) return QMOE_OK;
+        const int rc = gemm_dense_launch(dense_fmt, dense_xdt, dense, (hipStream_t)stream);
+        dense.count = 0;
+        return rc;
+    };
     for (int i = 0; i < count; ++i) {
         const qmoe_linear_problem& p = problems[i];
-        const bool ok = p.tokens == 1 && (uintptr_t)p.x % dtype_size(p.x_dtype) == 0 &&
-                        (uintptr_t)p.y % dtype_size(p.y_dtype) == 0 && stream_supported(p.fmt, p.w, p.n, p.k, p.x, p.x_dtype);
-        if (ok && args.count && args.p[0].fmt != p.fmt) {  // one packed format per launch
-            int rc = stream_launch(args, (hipStream_t)stream);
-            if (rc) return rc;
-            args.count = 0;
-        }
-        if (ok) {
+        const bool aligned = (uintptr_t)p.x % dtype_size(p.x_dtype) == 0 && (uintptr_t)p.y % dtype_size(p.y_dtype) == 0;
+        const bool streams = aligned && p.tokens == 1 && stream_supported(p.fmt, p.w, p.n, p.k, p.x, p.x_dtype);
+        const bool tiles = aligned && p.tokens >= 2 && gemm_supported(p.fmt, p.w, 0, p.n, p.k, p.x, p.x_dtype, p.k);
+        int rc;
+        if (streams) {
+            if ((rc = flush_dense())) return rc;
+            if (args.count && (args.p[0].fmt != p.fmt || args.count == STREAM_MAX_PROBLEMS) && (rc = flush_stream())) return rc;
             args.p[args.count++] = StreamProblem{(const uint8_t*)p.w, nullptr, p.x, p.y, p.n, p.k, p.fmt, 0,
                                                  p.x_dtype, p.y_dtype, 0, 0};
-        }
-        if (args.count == STREAM_MAX_PROBLEMS || (!ok && args.count) || (i == count - 1 && args.count)) {
-            int rc = stream_launch(args, (hipStream_t)stream);
-            if (rc) return rc;
-            args.count = 0;
-        }
-        if (!ok) {
-            int rc = linear_impl(p.w, p.fmt, p.n, p.k, p.x, p.x_dtype, p.tokens, p.y, p.y_dtype, (hipStream_t)stream);
-            if (rc) return rc;
+        } else if (tiles) {
+            if ((rc = flush_stream())) return rc;
+            if (dense.count && (dense_fmt != p.fmt || dense_xdt != p.x_dtype || dense.tokens != p.tokens ||
+                                dense.count == GEMM_MAX_PROBLEMS) && (rc = flush_dense())) return rc;
+            dense_fmt = p.fmt;
+            dense_xdt = p.x_dtype;
+            dense.tokens = p.tokens;
+            dense.p[dense.count++] = GemmDenseProblem{(const uint8_t*)p.w, p.x, p.y, p.n, p.k, p.y_dtype, 0};
+        } else {
+            if ((rc = flush_stream()) || (rc = flush_dense())) return rc;
+            if ((rc = linear_impl(p.w, p.fmt, p.n, p.k, p.x, p.x_dtype, p.tokens, p.y, p.y_dtype, (hipStream_t)stream))) return rc;
         }
     }
+    int rc;
+    if ((rc = flush_stream()) || (rc = flush_dense())) return rc;
     return QMOE_OK;
 }
 
