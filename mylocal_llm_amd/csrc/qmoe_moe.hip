@@ -70,6 +70,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
     const int assignments = tokens * k;
     int* expert_offset = (int*)(selection + (size_t)n_experts * words);
     for (int i = tid; i < n_experts * words; i += PLAN_THREADS) selection[i] = 0u;
+    if (tid == 0) *status = 0;
     __syncthreads();
     bool bad = false;
     for (int a = tid; a < assignments; a += PLAN_THREADS) {
@@ -214,17 +215,19 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     __shared__ float partial[4];
     __shared__ float sigmoid;
     const int t = blockIdx.x, tid = threadIdx.x;
-    if (tid == 0) {
-        // ascending sorted position == ascending expert id
-        int n = 0;
+    if (tid < 64) {
+        // ascending sorted position == ascending expert id; the first wave ranks the token's
+        // valid assignments among themselves (positions are unique)
+        const int p = tid < k ? pos_of[(size_t)t * k + tid] : -1;
+        const bool valid = p >= 0;
+        int rank = 0;
         for (int s = 0; s < k; ++s) {
-            int p = pos_of[(size_t)t * k + s];
-            if (p < 0) continue;
-            int j = n++;
-            while (j > 0 && order[j - 1] > p) { order[j] = order[j - 1]; --j; }
-            order[j] = p;
+            const int q = __builtin_amdgcn_readlane(p, s);
+            rank += q >= 0 && q < p;
         }
-        for (int s = n; s < k; ++s) order[s] = -1;
+        const int n = __popcll(__ballot(valid));
+        if (valid) order[rank] = p;
+        if (tid >= n && tid < 32) order[tid] = -1;
     }
     if (shared_out && shared_gate) {
         float a = 0.0f;
@@ -240,6 +243,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     }
     __syncthreads();
     const float sg = (shared_out && shared_gate) ? sigmoid : 1.0f;
+    if ((d & 3) == 0) {
+        // four columns per thread: the k loads of a column group travel together, the adds of
+        // each column stay in ascending expert order
+        for (int i = 4 * tid; i < d; i += 4 * 256) {
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int s = 0; s < k; ++s) {
+                const int p = order[s];
+                if (p >= 0) {
+                    const float4 v = *(const float4*)(terms + (size_t)p * d + i);
+                    acc.x = __fadd_rn(acc.x, v.x); acc.y = __fadd_rn(acc.y, v.y);
+                    acc.z = __fadd_rn(acc.z, v.z); acc.w = __fadd_rn(acc.w, v.w);
+                }
+            }
+            if (shared_out) {
+                const float4 v = *(const float4*)(shared_out + (size_t)t * d + i);
+                acc.x = add_product(acc.x, v.x, sg); acc.y = add_product(acc.y, v.y, sg);
+                acc.z = add_product(acc.z, v.z, sg); acc.w = add_product(acc.w, v.w, sg);
+            }
+            store_out(out, odt, (size_t)t * d + i, acc.x);
+            store_out(out, odt, (size_t)t * d + i + 1, acc.y);
+            store_out(out, odt, (size_t)t * d + i + 2, acc.z);
+            store_out(out, odt, (size_t)t * d + i + 3, acc.w);
+        }
+        return;
+    }
     for (int i = tid; i < d; i += 256) {
         float acc = 0.0f;
         for (int s = 0; s < k; ++s) {
@@ -343,7 +371,6 @@ static MoeWorkspace moe_layout(int tokens, int k, int n_experts, int d_model, in
     return w;
 }
 
-__global__ void clear_flags_kernel(int* a, int* b) { *a = 0; *b = 0; }
 
 template <int XDT>
 static void launch_gate_up(const qmoe_moe_args& a, const MoeWorkspace& L, char* ws, int max_active, bool xf,
@@ -508,7 +535,6 @@ int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_b
         weights = wout;
         ids = iout;
     }
-    hipLaunchKernelGGL(clear_flags_kernel, dim3(1), dim3(1), 0, s, (int*)(ws + L.n_active), (int*)(ws + L.status));
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, s, ids, weights, a.tokens, a.top_k,
                        b.n_experts, (int*)(ws + L.offsets), (int*)(ws + L.active), (int*)(ws + L.n_active),
                        (int*)(ws + L.sorted_token), (float*)(ws + L.sorted_weight), (int*)(ws + L.pos_of),
