@@ -166,6 +166,12 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
         }
 #pragma unroll
         for (int j = 0; j < NM; ++j) {
+            // Every dword of the unit becomes a value of its own here.  Without this, hipcc 7.2
+            // kept the unit in its 128-bit load tuples and, in the K-split variant, assigned a
+            // conversion result to a register of a tuple whose other bytes were still unread
+            // (wrong sums, caught by tests/test_gpu_linear.py).
+#pragma unroll
+            for (int i = 0; i < U::RAW; ++i) asm volatile("" : "+v"(raw[j][i]));
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
                 // the eight weights of step s only: the rest of the unit's decode is dead code

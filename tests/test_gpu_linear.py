@@ -135,6 +135,31 @@ def test_linear_batch_equals_separate_calls(cuda, tokens):
         assert rel_l2(out.cpu().numpy(), R.linear(xh, *triple(host))) <= 2e-5 <= REL_L2
 
 
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("tokens,dtype", [(5, "f32"), (40, "f32"), (17, "f16"), (33, "bf16")])
+def test_linear_batch_token_batches_long_rows(cuda, fmt, tokens, dtype):
+    """Token batches through one batched launch: rows of 8192 and 14336 columns (split over the
+    waves of a workgroup), a short matrix beside them, row counts that are not multiples of the
+    row tiles, token counts that end in a partly filled tile, all activation types."""
+    announce("linear batch long rows", fmt, tokens, dtype)
+    shapes = [(160, 8192), (100, 1024), (72, 14336), (16, 4096)]
+    hosts = [synthetic.packed_weight(fmt, shp, 700 + i) for i, shp in enumerate(shapes)]
+    ws = [upload(w, cuda) for w in hosts]
+    xs_host = [synthetic.activations((tokens, k), 800 + i) for i, (_, k) in enumerate(shapes)]
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    xs = [torch.from_numpy(x).to(cuda).to(tdt) for x in xs_host]
+    outs = quantized_linear_batch(list(zip(xs, ws)))
+    for out, x, host, (n, _) in zip(outs, xs, hosts, shapes):
+        assert out.shape == (tokens, n) and out.dtype == tdt
+        want = R.linear(x.float().cpu().numpy(), *triple(host))
+        if dtype == "f32":
+            assert rel_l2(out.cpu().numpy(), want) <= 2e-5 <= REL_L2
+        else:
+            scale = max(1.0, float(np.abs(want).max()))
+            tol = 2e-3 if dtype == "f16" else BF16_MAX_ABS
+            assert np.abs(out.float().cpu().numpy() - want).max() <= tol * scale
+
+
 @pytest.mark.parametrize("gf,uf", [("Q8_0", "Q8_0"), ("Q5_K", "Q4_K"), ("Q6_K", "Q6_K"), ("Q5_K", "Q5_K"), ("BF16", "Q8_0")])
 @pytest.mark.parametrize("m", [1, 3, 16])
 def test_swiglu_fused_matches_oracle_and_unfused(cuda, gf, uf, m):
