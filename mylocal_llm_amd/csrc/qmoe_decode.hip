@@ -469,7 +469,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     d.fsh = r.fsh;
     // enough workgroups to fill the chip at one token; longer walks (activations reused) beyond
     const long want = (long)a.tokens * b.d_model / 2048;
-    d.rows_per_wave = want >= 8 ? 8 : want >= 4 ? 4 : 2;
+    d.rows_per_wave = want >= 8 ? 8 : want >= 4 ? 4 : want >= 2 ? 2 : 1;
     const int rows_per_wg = 4 * d.rows_per_wave;
     const dim3 dgrid((b.d_model + rows_per_wg - 1) / rows_per_wg, a.tokens), dblock(256);
     const int lpe = b.d_ff >> 7;
