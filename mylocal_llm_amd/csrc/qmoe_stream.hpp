@@ -356,8 +356,9 @@ template <int FMT, bool PAIR> struct RowRegs {
     uint32_t b[PAIR ? Unit64<FMT>::RAW : 1];
 };
 
-// Rows of `LR` lanes each (64/LR rows per wave and step); WR waves share one row; PD rows
-// are requested ahead of the one being reduced.
+// Rows of `LR` lanes each (64/LR rows per wave and step); WR waves share one row (the
+// workgroup's four waves then work on 4/WR rows at a time); PD rows are requested ahead of
+// the one being reduced.
 template <int FMT, bool PAIR, int LR, int WR, int PD>
 __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* partial, float* xs, int& staged,
                                                float (&xr)[64], float (&aux)[8], int& xgroup) {
@@ -365,9 +366,10 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int units = p.k >> 6;
     const int64_t rb = row_bytes_dev(FMT, p.k);
-    constexpr int RPW = 64 / LR;                 // rows per wave step
-    const int sub = lane / LR;                   // which of the wave's rows this lane works on
-    const int u = (WR > 1 ? wave * 64 : 0) + (lane % LR);
+    constexpr int RPW = WR > 1 ? STREAM_WAVES / WR : 64 / LR;  // rows per step of a wave (of the workgroup if WR > 1)
+    const int sub = WR > 1 ? wave / WR : lane / LR;            // which of those rows this lane works on
+    const int part = WR > 1 ? wave % WR : 0;                   // which 4096-column part of the row
+    const int u = part * 64 + (lane % LR);
     const bool active = u < units;
     const int uu = active ? u : 0;
     // work items: groups of RPW rows; taken by waves (WR == 1) or by workgroups (WR > 1)
@@ -423,9 +425,12 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
             if (PAIR) {
                 const float up = group_sum<LR>(U::dot(buf[s].b, xr, aux));
                 if (WR == 1) v = silu_mul(g, up);
-                else if (lane == 63) { partial[(slot * 2) * WR + wave] = g; partial[(slot * 2 + 1) * WR + wave] = up; }
+                else if (lane == 63) {
+                    partial[((slot * RPW + sub) * 2) * WR + part] = g;
+                    partial[((slot * RPW + sub) * 2 + 1) * WR + part] = up;
+                }
             } else if (WR > 1) {
-                if (lane == 63) partial[slot * WR + wave] = g;
+                if (lane == 63) partial[(slot * RPW + sub) * WR + part] = g;
             }
             if (WR == 1) {
                 if ((lane % LR) == LR - 1 && row < p.n) store_out(p.y, p.ydt, row, v);
@@ -434,9 +439,9 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
                 ++slot;
                 if (slot == 32 || !more) {
                     __syncthreads();
-                    const int t = threadIdx.x;
-                    if (t < slot) {
-                        const int r2 = item - (slot - 1 - t) * workers;  // RPW == 1 when WR > 1
+                    const int t = threadIdx.x;  // entry t = step t / RPW of this flush, row t % RPW of the step
+                    const int r2 = (item - (slot - 1 - t / RPW) * workers) * RPW + t % RPW;
+                    if (t < slot * RPW && r2 < p.n) {
                         float sg = 0.f, su = 0.f;
 #pragma unroll
                         for (int wv = 0; wv < WR; ++wv) {

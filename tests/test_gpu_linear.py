@@ -160,6 +160,31 @@ def test_linear_batch_token_batches_long_rows(cuda, fmt, tokens, dtype):
             assert np.abs(out.float().cpu().numpy() - want).max() <= tol * scale
 
 
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("k", [512, 1024, 2048, 6144, 8192, 14336])
+def test_single_token_streaming_every_row_width(cuda, fmt, k):
+    """One token through the streaming kernel at every lane layout: 8 / 16 / 32 lanes per row,
+    two and four waves per row (6144 / 8192 and 14336 columns), alone and as a batch whose
+    problems have different widths; plus the fused gate/up pair at the same widths."""
+    announce("stream widths", fmt, k)
+    n = 72
+    hosts = [synthetic.packed_weight(fmt, (n, k), 40 + i) for i in range(2)]
+    x = synthetic.activations((1, k), 41)
+    xd = torch.from_numpy(x).to(cuda)
+    devs = [upload(w, cuda) for w in hosts]
+    for host, dev in zip(hosts, devs):
+        got = quantized_linear(xd, dev).cpu().numpy()
+        assert rel_l2(got, R.linear(x, *triple(host))) <= 2e-6 <= REL_L2
+    other = synthetic.packed_weight(fmt, (40, 4096), 44)
+    xo = synthetic.activations((1, 4096), 45)
+    outs = quantized_linear_batch([(xd, devs[0]), (torch.from_numpy(xo).to(cuda), upload(other, cuda)), (xd, devs[1])])
+    assert rel_l2(outs[0].cpu().numpy(), R.linear(x, *triple(hosts[0]))) <= 2e-6
+    assert rel_l2(outs[1].cpu().numpy(), R.linear(xo, *triple(other))) <= 2e-6
+    assert rel_l2(outs[2].cpu().numpy(), R.linear(x, *triple(hosts[1]))) <= 2e-6
+    h = quantized_swiglu(xd, devs[0], devs[1]).cpu().numpy()
+    assert rel_l2(h, R.swiglu(x, triple(hosts[0]), triple(hosts[1]))) <= 5e-6 <= REL_L2
+
+
 @pytest.mark.parametrize("gf,uf", [("Q8_0", "Q8_0"), ("Q5_K", "Q4_K"), ("Q6_K", "Q6_K"), ("Q5_K", "Q5_K"), ("BF16", "Q8_0")])
 @pytest.mark.parametrize("m", [1, 3, 16])
 def test_swiglu_fused_matches_oracle_and_unfused(cuda, gf, uf, m):

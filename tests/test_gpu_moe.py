@@ -335,3 +335,23 @@ def test_moe_token_batches_ragged_shapes(cuda, fmt, dtype):
     np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
     tol = 2e-5 if dtype == "f32" else 1e-3  # fp16 output rounding
     assert rel_l2(out.float().cpu().numpy(), want) <= tol <= REL_L2
+
+
+@pytest.mark.parametrize("tokens", [2, 7])
+def test_decode_path_with_more_experts_than_the_fused_launch_routes(cuda, tokens):
+    """1536 experts: wider than the rows the fused route + gate/up launch keeps in registers, so a
+    few tokens take the separate routing kernel and the device-side problem list."""
+    announce("moe decode wide router", tokens)
+    e, d, f, fsh, k = 1536, 256, 128, 256, 6
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh, ("Q8_0", "Q8_0", "Q8_0"), 2100)
+    hidden = synthetic.activations((tokens, d), 17, "bf16") * np.float32(3.0)
+    logits = synthetic.router_logits(tokens, e, 19)
+    assert not synthetic.has_topk_ties(logits, k)
+    want, want_w, want_ids = oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    dshared = tuple(upload(w, cuda) for w in shared)
+    out, w, ids = moe_step(torch.from_numpy(hidden).to(cuda), bank, k, logits=torch.from_numpy(logits).to(cuda),
+                           shared=dshared, shared_gate=torch.from_numpy(gate_vec).to(cuda), return_routing=True)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=2e-7)
+    assert rel_l2(out.cpu().numpy(), want) <= 2e-5 <= REL_L2
