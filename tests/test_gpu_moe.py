@@ -355,3 +355,45 @@ def test_decode_path_with_more_experts_than_the_fused_launch_routes(cuda, tokens
     np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
     np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=2e-7)
     assert rel_l2(out.cpu().numpy(), want) <= 2e-5 <= REL_L2
+
+
+@pytest.mark.parametrize("e,d,f,fsh,k,fmt,tokens,dtype", [
+    (8, 6144, 128, 256, 2, "Q8_0", 1, "f32"),     # rows of 6144 columns: two waves per row in the gate/up pairs
+    (8, 8192, 128, 128, 2, "Q8_0", 3, "bf16"),    # 8192 columns, three tokens, bf16 hidden states
+    (6, 10240, 128, 256, 2, "Q8_0", 2, "f32"),    # four waves per row
+    (8, 512, 1024, 1024, 4, "Q8_0", 2, "f32"),    # eight row parts per expert in the down kernel
+    (6, 512, 2048, 2048, 3, "Q8_0", 1, "f32"),    # sixteen row parts per expert
+    (8, 1024, 256, 512, 3, "BF16", 1, "f32"),     # BF16 bank
+    (8, 1024, 256, 512, 3, "BF16", 4, "bf16"),
+    (8, 1024, 256, 512, 3, "Q5_K", 9, "f16"),     # nine tokens: routing kernel + device-side list, fp16 hidden states
+    (8, 2048, 512, 0, 4, "Q6_K", 5, "f32"),       # no shared expert
+])
+def test_decode_shapes_lane_layouts_and_types(cuda, e, d, f, fsh, k, fmt, tokens, dtype):
+    """Decode-size steps across the lane layouts of the two kernels (row widths of the gate/up
+    stream, row parts of the down kernel), bank formats and hidden-state types."""
+    announce("moe decode shapes", e, d, f, fsh, k, fmt, tokens, dtype)
+    has_shared = fsh > 0
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh if has_shared else 256, (fmt, fmt, fmt), 3100)
+    # exact in bf16 and fp32 (fp16 rounds); the synthetic Q5_K scales / minima make outputs large,
+    # so those inputs are kept small enough for fp16 outputs
+    hidden = synthetic.activations((tokens, d), 23, "bf16") * np.float32(2.0 if fmt != "Q5_K" else 2.0 ** -6)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    hd = torch.from_numpy(hidden).to(cuda).to(tdt)
+    hidden = hd.float().cpu().numpy()
+    logits = synthetic.router_logits(tokens, e, 29)
+    assert not synthetic.has_topk_ties(logits, k)
+    ef = lambda i, rows: R.expert_ffn(rows, triple(gate.select_outer(i)), triple(up.select_outer(i)), triple(down.select_outer(i)))
+    if has_shared:
+        want, _, want_ids = R.moe_forward(hidden, logits, k, e, ef, tuple(triple(w) for w in shared), gate_vec)
+    else:
+        want_w, want_ids = R.router_topk(logits, k, renormalize=True, floor=2.0 ** -14)
+        want = R.experts_forward(hidden, want_w, want_ids, e, ef)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    kwargs = dict(shared=tuple(upload(w, cuda) for w in shared), shared_gate=torch.from_numpy(gate_vec).to(cuda)) if has_shared else {}
+    out, _, ids = moe_step(hd, bank, k, logits=torch.from_numpy(logits).to(cuda), return_routing=True, **kwargs)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    if dtype == "f32":
+        assert rel_l2(out.cpu().numpy(), want) <= 2e-5 <= REL_L2
+    else:
+        scale = max(1.0, float(np.abs(want).max()))
+        assert np.abs(out.float().cpu().numpy() - want).max() <= (2e-3 if dtype == "f16" else BF16_MAX_ABS) * scale
