@@ -3,8 +3,11 @@
 Mirrors ``PackedGGUFWeight`` of the reference (mini_llm/ops/quantized_weight.py:44-99):
 validation of shape / block alignment / byte count, a flat uint8 *view* of the caller's
 buffer (an mmap stays the owner), and zero-copy ``select_outer``.  Constructing it never
-materialises a floating-point matrix.  Decoding happens on the device only
-(``DevicePackedGGUFWeight.dequantize``); this package has no host decoder.
+materialises a floating-point matrix.  Decoding happens on the device only: the
+``*_reference`` methods of the reference's container (mini_llm/ops/quantized_weight.py:101-250,
+NumPy decoders there) keep their names, arguments and errors here but upload the packed rows
+they need and run the device decoder / linear; this package has no host decoder, and they
+raise without a HIP device.
 """
 from dataclasses import dataclass
 import math
@@ -80,3 +83,61 @@ class PackedGGUFWeight:
         row_bytes = self.nbytes // self.shape[0]
         return PackedGGUFWeight(self.data[start * row_bytes:stop * row_bytes],
                                 (stop - start, self.shape[1]), self.quant_type)
+
+    # ---- the reference's host helpers, computed on the device --------------------------------
+    @staticmethod
+    def _reference_tile_rows(tile_rows):
+        if isinstance(tile_rows, (bool, np.bool_)) or not isinstance(tile_rows, (int, np.integer)) or tile_rows <= 0:
+            raise ValueError("tile_rows must be a positive integer")
+        return int(tile_rows)
+
+    def _device_matrix(self, data, rows):
+        from .quantized_linear import packed_to_device
+        return packed_to_device(PackedGGUFWeight(data, (rows, self.shape[-1]), self.quant_type))
+
+    def dequantize_reference(self):
+        """fp32 ndarray of ``shape``, bit-identical to quantized_weight.py:151-250 (device decoder)."""
+        rows = math.prod(self.shape[:-1])
+        dense = self._device_matrix(self.data, rows).dequantize()
+        return dense.cpu().numpy().reshape(self.shape)
+
+    def dequantize_rows_reference(self, indices, *, tile_rows=32):
+        """Selected rows of a matrix, order and duplicates preserved (quantized_weight.py:101-125);
+        only the requested rows are uploaded and decoded, ``tile_rows`` of them at a time."""
+        if len(self.shape) != 2:
+            raise ValueError("selected rows require a matrix; select_outer first")
+        tile_rows = self._reference_tile_rows(tile_rows)
+        indices = np.asarray(indices)
+        if indices.ndim != 1 or indices.dtype.kind not in "iu":
+            raise ValueError("indices must be a one-dimensional integer array")
+        if np.any(indices >= self.shape[0]) or np.any(indices < 0):
+            raise IndexError("packed row index out of range")
+        result = np.empty((len(indices), self.shape[1]), dtype=np.float32)
+        raw = self.data.reshape(self.shape[0], self.nbytes // self.shape[0])
+        for start in range(0, len(indices), tile_rows):
+            selected = indices[start:start + tile_rows]
+            tile = self._device_matrix(np.ascontiguousarray(raw[selected]), len(selected))
+            result[start:start + len(selected)] = tile.dequantize().cpu().numpy()
+        return result
+
+    def matvec_reference(self, vector, *, tile_rows=32):
+        """fp32 ``W @ vector`` (quantized_weight.py:133-149): packed rows go to the device
+        ``tile_rows`` at a time and through the single-token linear."""
+        if len(self.shape) != 2:
+            raise ValueError("matvec requires a matrix; select_outer first")
+        tile_rows = self._reference_tile_rows(tile_rows)
+        vector = np.asarray(vector, dtype=np.float32)
+        if vector.shape != (self.shape[1],):
+            raise ValueError("vector shape must equal (matrix columns,)")
+        import torch
+        from .quantized_linear import quantized_linear
+        result = np.empty(self.shape[0], dtype=np.float32)
+        row_bytes = self.nbytes // self.shape[0]
+        x = None
+        for start in range(0, self.shape[0], tile_rows):
+            end = min(start + tile_rows, self.shape[0])
+            tile = self._device_matrix(self.data[start * row_bytes:end * row_bytes], end - start)
+            if x is None:
+                x = torch.from_numpy(np.ascontiguousarray(vector)[None]).to(tile.data.device)
+            result[start:end] = quantized_linear(x, tile).cpu().numpy()[0]
+        return result
