@@ -234,12 +234,16 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
             const size_t pos = (size_t)(start + tk);
             if (PAIR) {
                 if (rows[0] < a.n) {
-                    // SwiGLU, left as two bf16 terms for the down step's A operand
+                    // SwiGLU, left as two bf16 terms for the down step's A operand when a second array is given
                     const float v = silu_mul(acc[0][mt][i], acc[NM - 1][mt][i]);
-                    const uint16_t hi = float_to_bf16_bits(v);
-                    const uint16_t lo = float_to_bf16_bits(v - __uint_as_float((uint32_t)hi << 16));
-                    ((uint16_t*)a.out0)[pos * a.n + rows[0]] = hi;
-                    ((uint16_t*)a.out1)[pos * a.n + rows[0]] = lo;
+                    if (a.out1) {
+                        const uint16_t hi = float_to_bf16_bits(v);
+                        const uint16_t lo = float_to_bf16_bits(v - __uint_as_float((uint32_t)hi << 16));
+                        ((uint16_t*)a.out0)[pos * a.n + rows[0]] = hi;
+                        ((uint16_t*)a.out1)[pos * a.n + rows[0]] = lo;
+                    } else {
+                        store_out(a.out0, a.out_dt, pos * a.n + rows[0], v);  // a caller's SwiGLU output
+                    }
                 }
             } else {
 #pragma unroll

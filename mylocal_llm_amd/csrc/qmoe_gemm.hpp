@@ -24,8 +24,8 @@ struct GemmArgs {
     const int* chunk_count;
     const int* n_chunks;
     int dense_tokens;
-    // pair: SwiGLU output as bf16 hi / lo [positions, n]; else fp32 [positions, n], multiplied
-    // by scale[position] when scale is given
+    // pair: SwiGLU output as bf16 hi / lo [positions, n] (out1 given) or in out_dt (out1 null);
+    // else [positions, n] in out_dt, or fp32 multiplied by scale[position] when scale is given
     void* out0;
     void* out1;
     const float* scale;

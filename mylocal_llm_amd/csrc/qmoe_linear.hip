@@ -213,6 +213,19 @@ int swiglu_impl(const void* gate, int gf, const void* up, int uf, int f, int k, 
         args.p[0] = StreamProblem{(const uint8_t*)gate, (const uint8_t*)up, x, h, f, k, gf, 0, xdt, hdt, 0, 0};
         return stream_launch(args, s);
     }
+    if (tokens >= 2 && gf == uf && gemm_supported(gf, gate, 0, f, k, x, xdt, k) && gemm_supported(uf, up, 0, f, k, x, xdt, k)) {
+        GemmArgs g{};  // token batch: gate and up rows multiplied together on MFMA
+        g.w = (const uint8_t*)gate;
+        g.w2 = (const uint8_t*)up;
+        g.n = f;
+        g.k = k;
+        g.a0 = x;
+        g.a_stride = k;
+        g.dense_tokens = tokens;
+        g.out0 = h;
+        g.out_dt = hdt;
+        return gemm_launch(gf, true, xdt, g, (tokens + GEMM_CHUNK - 1) / GEMM_CHUNK, s);
+    }
     const bool xf = x_fast(x, xdt, k);
     const bool gfast = xf && rows_fast(gf, gate, row_bytes(gf, k), k);
     const bool ufast = xf && rows_fast(uf, up, row_bytes(uf, k), k);

@@ -196,7 +196,8 @@ def test_swiglu_fused_matches_oracle_and_unfused(cuda, gf, uf, m):
     dg, du = upload(gate, cuda), upload(up, cuda)
     xd = torch.from_numpy(x).to(cuda)
     got = quantized_swiglu(xd, dg, du).cpu().numpy()
-    assert rel_l2(got, want) <= 5e-6 <= REL_L2
+    # token batches of one format multiply on MFMA with 16-bit operand splits
+    assert rel_l2(got, want) <= (5e-6 if m == 1 else 2e-5) <= REL_L2
     g, u = quantized_linear(xd, dg), quantized_linear(xd, du)
     unfused = ((g / (1 + torch.exp(-g))) * u).cpu().numpy()
     np.testing.assert_allclose(got, unfused, rtol=3e-4, atol=2e-4 * np.abs(want).max())
