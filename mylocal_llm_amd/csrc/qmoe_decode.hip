@@ -45,6 +45,8 @@ struct DecodeRouteArgs {
     float* hs;                 // [T, Fsh]
     float floor_value;
     int renorm, n_experts, k, d, f, fsh, fmt, xdt, tokens, workers;
+    int shared_apart;          // the shared expert's gate/up is not in the problem list: its rows are
+                               // streamed once for all tokens by a phase of its own
 };
 
 // hidden[t] . g for the shared expert's admission gate, 2048 columns at a time: issue() only
@@ -133,10 +135,11 @@ __device__ __forceinline__ void route_token(const DecodeRouteArgs& a, int t, boo
 // Entry j of token t's part of the problem list: the gate/up pair of its j-th expert in
 // ascending id (j < k) or of the shared expert (j == k).
 __device__ __forceinline__ StreamProblem decode_problem(const DecodeRouteArgs& a, int t, int j, int64_t e) {
+    const bool shared_listed = a.shared_gate_w && !a.shared_apart;
     const int k = a.k;
     const int units = a.d >> 6;
     const int rpw = 64 / lanes_per_row(a.d);
-    const int items_r = (a.f + rpw - 1) / rpw, items_s = a.shared_gate_w ? (a.fsh + rpw - 1) / rpw : 0;
+    const int items_r = (a.f + rpw - 1) / rpw, items_s = shared_listed ? (a.fsh + rpw - 1) / rpw : 0;
     const int wide = units > 64 ? STREAM_WAVES : 1;
     const int64_t xbytes = (int64_t)a.d * (a.xdt == QMOE_DT_F32 ? 4 : 2);
     const long cursor = ((long)t * ((long)k * items_r + items_s) + (long)j * items_r) * wide;
@@ -175,18 +178,42 @@ __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs 
     const int t = blockIdx.x, lane = threadIdx.x;
     route_token<64>(a, t, true, sid, [] {});
     __syncthreads();
-    const int per_token = a.k + (a.shared_gate_w ? 1 : 0);
+    const int per_token = a.k + (a.shared_gate_w && !a.shared_apart ? 1 : 0);
     if (lane == 0 && t == 0) *a.problem_count = a.tokens * per_token;
     if (lane < per_token) a.problems[(size_t)t * per_token + lane] = decode_problem(a, t, lane, lane < a.k ? sid[lane] : 0);
+}
+
+// The shared expert's gate/up rows for all tokens of the step: tokens are staged in LDS in groups
+// (as many padded rows as fit), every workgroup stages the same group, and the rows are streamed
+// once per group instead of once per token.  Workgroup-uniform; ends with the LDS free again.
+template <int FMT>
+__device__ __forceinline__ void shared_pairs_phase(const DecodeRouteArgs& a, float* xs) {
+    const int stripe = a.d + 4 * (a.d >> 6);
+    const int fit = STREAM_XS_FLOATS / stripe;
+    const int wave = threadIdx.x >> 6;
+    for (int t0 = 0; t0 < a.tokens; t0 += fit) {
+        const int groups = a.tokens - t0 < fit ? a.tokens - t0 : fit;
+        __syncthreads();
+        for (int g = 0; g < groups; ++g)
+            for (int i = 4 * threadIdx.x; i < a.d; i += 4 * STREAM_THREADS)
+                *(float4*)(xs + g * stripe + StagedX::at(i)) = load_x4(a.hidden, a.xdt, (t0 + g) * a.d + i);
+        __syncthreads();
+        stream_rows_many_x<FMT, true, Prefetch<FMT, true>::DEPTH>(a.shared_gate_w, a.shared_up_w, a.fsh, a.d, xs, stripe, groups,
+                                                                 a.hs + (size_t)t0 * a.fsh, a.fsh,
+                                                                 blockIdx.x * STREAM_WAVES + wave, gridDim.x * STREAM_WAVES);
+    }
+    __syncthreads();
 }
 
 // The streaming engine over a problem list that lives in device memory.
 template <int FMT, bool PAIR>
 __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const StreamProblem* __restrict__ list,
-                                                                       const int* __restrict__ count) {
+                                                                       const int* __restrict__ count,
+                                                                       const DecodeRouteArgs a) {
     __shared__ float partial[32 * 2 * 4];
     __shared__ StreamProblem staged[LIST_STAGE];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
+    if (a.shared_apart) shared_pairs_phase<FMT>(a, xs);
     const int n = *count;
     // descriptors are fetched a stage at a time by the whole workgroup, not one dependent
     // load per problem
@@ -427,6 +454,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     r.tokens = a.tokens;
     r.workers = grid * STREAM_WAVES;
     int rc;
+    r.shared_apart = 0;
     const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.top_k + 1 <= FUSED_MAX_SLOTS && b.d_model <= 4096 &&
                        (!a.logits || b.n_experts <= FUSED_MAX_EXPERTS);
     if (fused) {
@@ -439,10 +467,11 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
         }
         if ((rc = check_launch("qmoe_moe_forward(route + gate/up)"))) return rc;
     } else {
+    r.shared_apart = has_shared && b.d_model <= 4096 && a.tokens >= 2;
     hipLaunchKernelGGL(decode_route_kernel, dim3(a.tokens), dim3(64), 0, s, r);
     if ((rc = check_launch("qmoe_moe_forward(route)"))) return rc;
 #define QMOE_LIST(F) hipLaunchKernelGGL((stream_list_kernel<F, true>), dim3(grid), dim3(STREAM_THREADS), 0, s, \
-                                        (const StreamProblem*)w.problems, (const int*)w.problem_count)
+                                        (const StreamProblem*)w.problems, (const int*)w.problem_count, r)
     switch (b.gate_fmt) {
     case QMOE_FMT_Q8_0: QMOE_LIST(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_LIST(QMOE_FMT_Q6_K); break;

@@ -589,6 +589,59 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
     }
 }
 
+// One matrix (or gate/up pair) of rows of up to 4096 columns multiplied with SEVERAL activation
+// rows that lie in LDS stripes (padded layout, `stripe` floats apart): every row is streamed
+// once and reduced against each staged activation row in turn; results go to fp32
+// y[g * ystride + row].  The caller is worker `me` of `W`; item i belongs to worker i mod W.
+template <int FMT, bool PAIR, int PD>
+__device__ __forceinline__ void stream_rows_many_x(const uint8_t* w, const uint8_t* w2, int n, int k, const float* xs,
+                                                   int stripe, int groups, float* y, int64_t ystride, int me, int W) {
+    using U = Unit64<FMT>;
+    const int lane = threadIdx.x & 63;
+    const int lr = lanes_per_row(k), units = k >> 6;
+    const int u = lane & (lr - 1);
+    const bool active = u < units;
+    const int uu = active ? u : 0;
+    const int rpw = 64 / lr;
+    const int items = (n + rpw - 1) / rpw;
+    const int64_t rb = row_bytes_dev(FMT, k);
+    int item = me;
+    if (item >= items) return;
+    RowRegs<FMT, PAIR> buf[PD + 1];
+    auto fetch = [&](int it, RowRegs<FMT, PAIR>& r) {
+        const int row = it * rpw + lane / lr;
+        const int64_t rr = row < n ? row : n - 1;
+        U::load_w(w + rr * rb, uu, r.a);
+        if (PAIR) U::load_w(w2 + rr * rb, uu, r.b);
+    };
+#pragma unroll
+    for (int j = 0; j < PD; ++j)
+        if (item + j * W < items) fetch(item + j * W, buf[j]);
+    bool done = false;
+    while (!done) {
+#pragma unroll
+        for (int s = 0; s <= PD; ++s) {
+            if (!done) {
+                if (item + PD * W < items) fetch(item + PD * W, buf[(s + PD) % (PD + 1)]);
+                const int row = item * rpw + lane / lr;
+                for (int g = 0; g < groups; ++g) {
+                    float xr[64], aux[8];
+                    U::load_x(StagedX{xs + g * stripe}, uu, xr, aux);
+                    float a = U::dot(buf[s].a, xr, aux);
+                    a = group_sum_rt(active ? a : 0.f, lr);
+                    if (PAIR) {
+                        float b = U::dot(buf[s].b, xr, aux);
+                        a = silu_mul(a, group_sum_rt(active ? b : 0.f, lr));
+                    }
+                    if (u == lr - 1 && row < n) y[g * ystride + row] = a;
+                }
+                item += W;
+                if (item >= items) done = true;
+            }
+        }
+    }
+}
+
 // Rows requested ahead: bounded by the 256-VGPR budget (a BF16 unit is 32 dwords per row).
 template <int FMT, bool PAIR> struct Prefetch {
     static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (FMT == QMOE_FMT_Q8_0 ? (PAIR ? 1 : 2) : (PAIR ? 1 : 4));
