@@ -29,13 +29,17 @@ __device__ __forceinline__ float half_bits_to_float(uint32_t h) {
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
 
 // Loads that only assume the alignment the format guarantees.
-__device__ __forceinline__ uint32_t ld_u16(const uint8_t* p) { return *(const uint16_t*)p; }
+__device__ __forceinline__ uint32_t ld_u16(const uint8_t* p) { return *(const __attribute__((address_space(1))) uint16_t*)p; }
 __device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t* p) {
     return ld_u16(p) | (ld_u16(p + 2) << 16);
 }
-__device__ __forceinline__ uint32_t ld_u32(const uint8_t* p) { return *(const uint32_t*)p; }
+__device__ __forceinline__ uint32_t ld_u32(const uint8_t* p) { return *(const __attribute__((address_space(1))) uint32_t*)p; }
 struct __attribute__((packed, aligned(4))) u32x4_a4 { uint32_t v[4]; };
-__device__ __forceinline__ u32x4_a4 ld_u32x4_a4(const uint8_t* p) { return *(const u32x4_a4*)p; }
+__device__ __forceinline__ u32x4_a4 ld_u32x4_a4(const uint8_t* p) {
+    typedef uint32_t V __attribute__((ext_vector_type(4), aligned(4)));
+    const V v = *(const __attribute__((address_space(1))) V*)p;
+    return u32x4_a4{{v[0], v[1], v[2], v[3]}};
+}
 
 __device__ __forceinline__ float sbyte(uint32_t word, int i) {
     return (float)(int)(int8_t)(word >> (8 * i));

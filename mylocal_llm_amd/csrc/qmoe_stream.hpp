@@ -36,9 +36,6 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-struct __attribute__((packed, aligned(2))) u32x4_a2 { uint32_t v[4]; };
-struct __attribute__((packed, aligned(2))) u32x2_a2 { uint32_t v[2]; };
-struct __attribute__((packed, aligned(2))) u32_a2 { uint32_t v; };
 
 __device__ __forceinline__ float ubyte_f(uint32_t w, int i) {
     // v_cvt_f32_ubyte{0..3}
@@ -83,10 +80,10 @@ template <> struct Unit64<QMOE_FMT_Q8_0> {
         const uint8_t* p = row + (size_t)u * 68;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            u32x4_a4 v = *(const u32x4_a4*)(p + 16 * i);
-            r[4 * i] = v.v[0]; r[4 * i + 1] = v.v[1]; r[4 * i + 2] = v.v[2]; r[4 * i + 3] = v.v[3];
+            const u32x4_t v = ldg_u32x4<4>(p + 16 * i);
+            r[4 * i] = v[0]; r[4 * i + 1] = v[1]; r[4 * i + 2] = v[2]; r[4 * i + 3] = v[3];
         }
-        r[16] = *(const uint32_t*)(p + 64);
+        r[16] = ldg<uint32_t>(p + 64);
     }
     __device__ __forceinline__ static float dot(const uint32_t* r, const float* xr, const float*) {
         const float d0 = half_bits_to_float(r[0] & 0xFFFFu), d1 = half_bits_to_float(r[8] >> 16);
@@ -136,14 +133,14 @@ template <> struct Unit64<QMOE_FMT_Q6_K> {
     __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
         const uint8_t* b = row + (size_t)(u >> 2) * 210;
         const int h = (u >> 1) & 1, c = u & 1;
-        u32x4_a2 la = *(const u32x4_a2*)(b + 64 * h + 16 * c);
-        u32x4_a2 lb = *(const u32x4_a2*)(b + 64 * h + 32 + 16 * c);
-        u32x4_a2 hq = *(const u32x4_a2*)(b + 128 + 32 * h + 16 * c);
-        u32x2_a2 sc = *(const u32x2_a2*)(b + 192 + 8 * h);
+        const u32x4_t la = ldg_u32x4<2>(b + 64 * h + 16 * c);
+        const u32x4_t lb = ldg_u32x4<2>(b + 64 * h + 32 + 16 * c);
+        const u32x4_t hq = ldg_u32x4<2>(b + 128 + 32 * h + 16 * c);
+        const u32x2_t sc = ldg_u32x2<2>(b + 192 + 8 * h);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { r[i] = la.v[i]; r[4 + i] = lb.v[i]; r[8 + i] = hq.v[i]; }
+        for (int i = 0; i < 4; ++i) { r[i] = la[i]; r[4 + i] = lb[i]; r[8 + i] = hq[i]; }
         // the four sub-block scales of this unit are bytes c, c+2, c+4, c+6 of the half's eight
-        const uint32_t s0 = sc.v[0] >> (8 * c), s1 = sc.v[1] >> (8 * c);
+        const uint32_t s0 = sc[0] >> (8 * c), s1 = sc[1] >> (8 * c);
         r[12] = (s0 & 0xFFu) | ((s0 >> 8) & 0xFF00u);         // scales of quarters 0, 1
         r[13] = (s1 & 0xFFu) | ((s1 >> 8) & 0xFF00u);         // scales of quarters 2, 3
         r[14] = ld_u16(b + 208);
@@ -208,13 +205,13 @@ template <> struct Unit64<QMOE_FMT_Q5_K> {
     __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
         const uint8_t* b = row + (size_t)(u >> 2) * 176;
         const int c = u & 3;
-        const uint4 hdr = *(const uint4*)b;
+        const uint4 hdr = ldg<uint4>(b);
         r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
-        const uint2 qh = *(const uint2*)(b + 16 + 8 * c);
+        const uint2 qh = ldg<uint2>(b + 16 + 8 * c);
         r[4] = qh.x; r[5] = qh.y;
 #pragma unroll
         for (int g2 = 0; g2 < 4; ++g2) {
-            const uint2 qs = *(const uint2*)(b + 48 + 32 * g2 + 8 * c);
+            const uint2 qs = ldg<uint2>(b + 48 + 32 * g2 + 8 * c);
             r[6 + 2 * g2] = qs.x; r[7 + 2 * g2] = qs.y;
         }
     }
@@ -277,10 +274,10 @@ template <> struct Unit64<QMOE_FMT_BF16> {
         }
     }
     __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
-        const uint4* p = (const uint4*)(row + (size_t)u * 128);
+        const uint8_t* p = row + (size_t)u * 128;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint4 v = p[i];
+            const uint4 v = ldg<uint4>(p + 16 * i);
             r[4 * i] = v.x; r[4 * i + 1] = v.y; r[4 * i + 2] = v.z; r[4 * i + 3] = v.w;
         }
     }
@@ -539,9 +536,14 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
         U::load_w(c_w + rr * rb, uu, r.a);
         if (PAIR) U::load_w(c_w2 + rr * rb, uu, r.b);
     };
+    // Every fetch is issued on every path (past the end the wave's last item is requested
+    // again): the number of loads in flight behind the rows about to be reduced is then the
+    // same whichever way the branches go, and the wait before the reduction can leave them
+    // in flight.
+    const int last = end - 1 - (end - 1 - g) % step;
+    auto bounded = [&](int gi) { return gi < end ? gi : last; };
 #pragma unroll
-    for (int j = 0; j < PD; ++j)
-        if (g + j * step < end) fetch(g + j * step, buf[j], bp[j], bi[j]);
+    for (int j = 0; j < PD; ++j) fetch(bounded(g + j * step), buf[j], bp[j], bi[j]);
     float xr[64], aux[8];
     int xgroup = -1;
     bool done = false;
@@ -550,7 +552,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
         for (int s = 0; s <= PD; ++s) {
             if (!done) {
                 const int nb = (s + PD) % (PD + 1);
-                if (g + PD * step < end) fetch(g + PD * step, buf[nb], bp[nb], bi[nb]);
+                fetch(bounded(g + PD * step), buf[nb], bp[nb], bi[nb]);
                 const StreamProblem& p = probs[bp[s]];
                 const int pk = uniform(p.k), pn = uniform(p.n), pg = uniform(p.xgroup);
                 const int lr = lanes_per_row(pk), units = pk >> 6;
@@ -642,9 +644,11 @@ __device__ __forceinline__ void stream_rows_many_x(const uint8_t* w, const uint8
     }
 }
 
-// Rows requested ahead: bounded by the 256-VGPR budget (a BF16 unit is 32 dwords per row).
+// Rows requested ahead (measured: with eight waves per CU one row ahead keeps the memory system
+// busy, and more only lengthens the queues in the vector cache; BF16 units are a cache line
+// per lane and do best with none).
 template <int FMT, bool PAIR> struct Prefetch {
-    static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? (PAIR ? 0 : 1) : (FMT == QMOE_FMT_Q8_0 ? (PAIR ? 1 : 2) : (PAIR ? 1 : 4));
+    static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? 0 : (FMT == QMOE_FMT_Q8_0 || PAIR) ? 1 : 2;
 };
 
 // A whole problem list held in LDS: first the single stream of all problems whose rows fit a
