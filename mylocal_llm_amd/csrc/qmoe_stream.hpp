@@ -506,7 +506,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
     // the problem the fetch side is in, held in scalar registers
     int cursor = -1, c_begin = 0, c_end = begin, c_n = 1, c_k = 64;
     const uint8_t *c_w = nullptr, *c_w2 = nullptr;
-    auto fetch = [&](int gi, RowRegs<FMT, PAIR>& r, int& rp, int& ri) {
+    auto fetch = [&](int gi, bool past, RowRegs<FMT, PAIR>& r, int& rp, int& ri) {
         if (gi >= c_end || cursor < 0) {
             // 64 range ends at a time: one LDS read and a ballot per hop
             ++cursor;
@@ -529,21 +529,21 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
         ri = gi - c_begin;
         const int lr = lanes_per_row(c_k), units = c_k >> 6;
         const int u = lane & (lr - 1);
-        const int uu = u < units ? u : 0;
+        const int uu = u < units && !past ? u : 0;
         const int row = ri * (64 / lr) + lane / lr;
-        const int64_t rr = row < c_n ? row : (c_n > 0 ? c_n - 1 : 0);
+        const int64_t rr = past ? 0 : row < c_n ? row : (c_n > 0 ? c_n - 1 : 0);
         const int64_t rb = row_bytes_dev(FMT, c_k);
         U::load_w(c_w + rr * rb, uu, r.a);
         if (PAIR) U::load_w(c_w2 + rr * rb, uu, r.b);
     };
-    // Every fetch is issued on every path (past the end the wave's last item is requested
-    // again): the number of loads in flight behind the rows about to be reduced is then the
-    // same whichever way the branches go, and the wait before the reduction can leave them
-    // in flight.
+    // Every fetch is issued on every path (past the end all lanes request the first bytes of
+    // the current matrix: one cache line): the number of loads in flight behind the rows about
+    // to be reduced is then the same whichever way the branches go, and the wait before the
+    // reduction can leave them in flight.
     const int last = end - 1 - (end - 1 - g) % step;
     auto bounded = [&](int gi) { return gi < end ? gi : last; };
 #pragma unroll
-    for (int j = 0; j < PD; ++j) fetch(bounded(g + j * step), buf[j], bp[j], bi[j]);
+    for (int j = 0; j < PD; ++j) fetch(bounded(g + j * step), g + j * step >= end, buf[j], bp[j], bi[j]);
     float xr[64], aux[8];
     int xgroup = -1;
     bool done = false;
@@ -552,7 +552,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
         for (int s = 0; s <= PD; ++s) {
             if (!done) {
                 const int nb = (s + PD) % (PD + 1);
-                fetch(bounded(g + PD * step), buf[nb], bp[nb], bi[nb]);
+                fetch(bounded(g + PD * step), g + PD * step >= end, buf[nb], bp[nb], bi[nb]);
                 const StreamProblem& p = probs[bp[s]];
                 const int pk = uniform(p.k), pn = uniform(p.n), pg = uniform(p.xgroup);
                 const int lr = lanes_per_row(pk), units = pk >> 6;
@@ -645,10 +645,10 @@ __device__ __forceinline__ void stream_rows_many_x(const uint8_t* w, const uint8
 }
 
 // Rows requested ahead (measured: with eight waves per CU one row ahead keeps the memory system
-// busy, and more only lengthens the queues in the vector cache; BF16 units are a cache line
-// per lane and do best with none).
+// busy, and more only lengthens the queues in the vector cache; BF16 units, a cache line per
+// lane, and gate/up pairs, two rows per step, do best with none).
 template <int FMT, bool PAIR> struct Prefetch {
-    static constexpr int DEPTH = FMT == QMOE_FMT_BF16 ? 0 : (FMT == QMOE_FMT_Q8_0 || PAIR) ? 1 : 2;
+    static constexpr int DEPTH = (FMT == QMOE_FMT_BF16 || PAIR) ? 0 : FMT == QMOE_FMT_Q8_0 ? 1 : 2;
 };
 
 // A whole problem list held in LDS: first the single stream of all problems whose rows fit a
