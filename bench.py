@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # (name, N, K) of the seven projections of one Llama-3-8B layer
 PROJECTIONS = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
                ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
-BLOCKS = {"Q8_0": (32, 34), "Q5_K": (256, 176), "Q6_K": (256, 210), "BF16": (1, 2)}
+BLOCKS = {"Q8_0": (32, 34), "Q5_K": (256, 176), "Q4_K": (256, 144), "Q6_K": (256, 210), "BF16": (1, 2)}
 
 
 def weight_bytes(fmt, n, k):
@@ -57,7 +57,7 @@ def device_blocks(torch, fmt, n, k, gen, device):
         blk[:, 0:192] = torch.randint(0, 256, (nb, 192), device=device, generator=gen, dtype=torch.uint8)
         blk[:, 192:208] = torch.randint(-64, 64, (nb, 16), device=device, generator=gen, dtype=torch.int8).view(torch.uint8)
         blk[:, 208:210] = scale(nb)
-    elif fmt == "Q5_K":
+    elif fmt in ("Q5_K", "Q4_K"):
         blk[:, 0:2] = scale(nb)
         blk[:, 2:4] = scale(nb)
         # any 12 bytes are a valid field of eight 6-bit (scale, min) pairs, uniform over 0..63
@@ -349,7 +349,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extras:
         extras = []
-        for fmt, tokens in (("Q6_K", 1), ("Q5_K", 1), ("BF16", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16)):
+        for fmt, tokens in (("Q6_K", 1), ("Q5_K", 1), ("Q4_K", 1), ("BF16", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16)):
             s = LayerStream(torch, lib, fmt, 8, tokens, device)
             w, m = time_steps(torch, s.step, max(3, args.steps // 4), 2)
             n = max(3, args.steps // 4)

@@ -385,7 +385,7 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
 
 // ---- host side ------------------------------------------------------------------------------------
 static bool stream_format(int fmt) {
-    return fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_BF16;
+    return fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_BF16;
 }
 
 // May this MoE step take the three-launch decode path?
@@ -398,7 +398,7 @@ bool decode_supported(const qmoe_moe_args& a, const void* h_ws) {
     const int lpe = b.d_ff >> 7;
     if (b.d_ff % 128 || (lpe & (lpe - 1)) || lpe > 16 || a.top_k * lpe > 48) return false;
     if (has_shared && (a.d_ff_shared % 128 || (a.d_ff_shared >> 7) > 16)) return false;
-    const bool kq = b.down_fmt == QMOE_FMT_Q6_K || b.down_fmt == QMOE_FMT_Q5_K;
+    const bool kq = b.down_fmt == QMOE_FMT_Q6_K || b.down_fmt == QMOE_FMT_Q5_K || b.down_fmt == QMOE_FMT_Q4_K;
     if (kq && (b.d_ff % 256 || (has_shared && a.d_ff_shared % 256))) return false;
     const int ga = b.gate_fmt == QMOE_FMT_Q8_0 ? 4 : b.gate_fmt == QMOE_FMT_Q6_K ? 2 : 16;
     const int da = b.down_fmt == QMOE_FMT_Q8_0 ? 4 : b.down_fmt == QMOE_FMT_Q6_K ? 2 : 16;
@@ -463,6 +463,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
         case QMOE_FMT_Q8_0: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q8_0>, fg, fb, 0, s, r); break;
         case QMOE_FMT_Q6_K: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q6_K>, fg, fb, 0, s, r); break;
         case QMOE_FMT_Q5_K: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q5_K>, fg, fb, 0, s, r); break;
+        case QMOE_FMT_Q4_K: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q4_K>, fg, fb, 0, s, r); break;
         default: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_BF16>, fg, fb, 0, s, r); break;
         }
         if ((rc = check_launch("qmoe_moe_forward(route + gate/up)"))) return rc;
@@ -476,6 +477,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     case QMOE_FMT_Q8_0: QMOE_LIST(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_LIST(QMOE_FMT_Q6_K); break;
     case QMOE_FMT_Q5_K: QMOE_LIST(QMOE_FMT_Q5_K); break;
+    case QMOE_FMT_Q4_K: QMOE_LIST(QMOE_FMT_Q4_K); break;
     default: QMOE_LIST(QMOE_FMT_BF16); break;
     }
 #undef QMOE_LIST
@@ -515,6 +517,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     case QMOE_FMT_Q8_0: QMOE_DOWN_F(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_DOWN_F(QMOE_FMT_Q6_K); break;
     case QMOE_FMT_Q5_K: QMOE_DOWN_F(QMOE_FMT_Q5_K); break;
+    case QMOE_FMT_Q4_K: QMOE_DOWN_F(QMOE_FMT_Q4_K); break;
     default: QMOE_DOWN_F(QMOE_FMT_BF16); break;
     }
 #undef QMOE_DOWN_F

@@ -335,6 +335,7 @@ int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, h
     case QMOE_FMT_Q8_0: QMOE_GEMM_F(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_GEMM_F(QMOE_FMT_Q6_K); break;
     case QMOE_FMT_Q5_K: QMOE_GEMM_F(QMOE_FMT_Q5_K); break;
+    case QMOE_FMT_Q4_K: QMOE_GEMM_F(QMOE_FMT_Q4_K); break;
     default: QMOE_GEMM_F(QMOE_FMT_BF16); break;
     }
 #undef QMOE_GEMM_F
@@ -379,6 +380,7 @@ int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     case QMOE_FMT_Q8_0: QMOE_DENSE_F(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_DENSE_F(QMOE_FMT_Q6_K); break;
     case QMOE_FMT_Q5_K: QMOE_DENSE_F(QMOE_FMT_Q5_K); break;
+    case QMOE_FMT_Q4_K: QMOE_DENSE_F(QMOE_FMT_Q4_K); break;
     default: QMOE_DENSE_F(QMOE_FMT_BF16); break;
     }
 #undef QMOE_DENSE_F

@@ -188,6 +188,7 @@ int smallm_launch(int fmt, const void* w, int n, int k, const void* x, int xdt, 
     case QMOE_FMT_Q8_0: smallm_launch_f<QMOE_FMT_Q8_0>(w, n, k, x, xdt, tokens, y, ydt, s); break;
     case QMOE_FMT_Q6_K: smallm_launch_f<QMOE_FMT_Q6_K>(w, n, k, x, xdt, tokens, y, ydt, s); break;
     case QMOE_FMT_Q5_K: smallm_launch_f<QMOE_FMT_Q5_K>(w, n, k, x, xdt, tokens, y, ydt, s); break;
+    case QMOE_FMT_Q4_K: smallm_launch_f<QMOE_FMT_Q4_K>(w, n, k, x, xdt, tokens, y, ydt, s); break;
     default: smallm_launch_f<QMOE_FMT_BF16>(w, n, k, x, xdt, tokens, y, ydt, s); break;
     }
     return check_launch("small-batch linear");

@@ -48,9 +48,9 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamA
 
 // ---- host side ---------------------------------------------------------------------------------
 bool stream_supported(int fmt, const void* w, int n, int k, const void* x, int xdt) {
-    if (!(fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_BF16)) return false;
+    if (!(fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_BF16)) return false;
     if (k % 64 || k > 256 * 64 || n < 1) return false;
-    if ((fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K) && (k % 256)) return false;
+    if ((fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q4_K) && (k % 256)) return false;
     const int align = fmt == QMOE_FMT_Q8_0 ? 4 : fmt == QMOE_FMT_Q6_K ? 2 : 16;
     if ((uintptr_t)w % align || row_bytes(fmt, k) % align) return false;
     return x_fast(x, xdt, k);
@@ -119,6 +119,7 @@ int stream_launch(StreamArgs& args, hipStream_t s) {
     case QMOE_FMT_Q8_0: QMOE_STREAM(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_STREAM(QMOE_FMT_Q6_K); break;
     case QMOE_FMT_Q5_K: QMOE_STREAM(QMOE_FMT_Q5_K); break;
+    case QMOE_FMT_Q4_K: QMOE_STREAM(QMOE_FMT_Q4_K); break;
     default: QMOE_STREAM(QMOE_FMT_BF16); break;
     }
 #undef QMOE_STREAM

@@ -10,6 +10,7 @@
 //   Q8_0  unit = 2 blocks            68 B  (4 x 16 B + 4 B)
 //   Q6_K  unit = quarter block       48 B + 8 B scales + 2 B d   (16-lane runs of 4 quarters)
 //   Q5_K  unit = quarter block       40 B + 16 B header          (8-lane runs of 8 groups)
+//   Q4_K  unit = quarter block       32 B + 16 B header
 //   BF16  unit = 64 elements        128 B
 #pragma once
 #include "qmoe_common.hpp"
@@ -262,6 +263,68 @@ template <> struct Unit64<QMOE_FMT_Q5_K> {
     __device__ __forceinline__ static int kstep(int u, int m) { return (u >> 2) * 256 + (u & 3) * 8 + 32 * m; }
 };
 
+// ---- Q4_K -----------------------------------------------------------------------------------
+// Q5_K without the fifth bit: unit u = block u/4, byte column c = u%4; element (group g, j) of
+// the unit is block element 32g + 8c + j.
+template <> struct Unit64<QMOE_FMT_Q4_K> {
+    static constexpr int RAW = 12, AUX = 8;
+    static constexpr int ROW_ALIGN = 16;
+    template <class X> __device__ __forceinline__ static void load_x(const X& x, int u, float* xr, float* aux) {
+        Unit64<QMOE_FMT_Q5_K>::load_x(x, u, xr, aux);
+    }
+    __device__ __forceinline__ static void load_w(const uint8_t* row, int u, uint32_t* r) {
+        const uint8_t* b = row + (size_t)(u >> 2) * 144;
+        const int c = u & 3;
+        const uint4 hdr = ldg<uint4>(b);
+        r[0] = hdr.x; r[1] = hdr.y; r[2] = hdr.z; r[3] = hdr.w;
+#pragma unroll
+        for (int g2 = 0; g2 < 4; ++g2) {
+            const uint2 qs = ldg<uint2>(b + 16 + 32 * g2 + 8 * c);
+            r[4 + 2 * g2] = qs.x; r[5 + 2 * g2] = qs.y;
+        }
+    }
+    __device__ __forceinline__ static float dot(const uint32_t* r, const float* xr, const float* aux) {
+        const float d = half_bits_to_float(r[0] & 0xFFFFu), dmin = half_bits_to_float(r[0] >> 16);
+        const uint32_t sc_lo = r[1] & 0x3F3F3F3Fu, mn_lo = r[2] & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (r[3] & 0x0F0F0F0Fu) | ((r[1] >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((r[3] >> 4) & 0x0F0F0F0Fu) | ((r[2] >> 2) & 0x30303030u);
+        float total = 0.f;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            float acc = 0.f;
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                const uint32_t qs = r[4 + 2 * (g >> 1) + m];
+                const uint32_t code = (g & 1) ? ((qs >> 4) & 0x0F0F0F0Fu) : (qs & 0x0F0F0F0Fu);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc += ubyte_f(code, j) * xr[8 * g + 4 * m + j];
+            }
+            const float sc = ubyte_f(g < 4 ? sc_lo : sc_hi, g & 3), mn = ubyte_f(g < 4 ? mn_lo : mn_hi, g & 3);
+            total += (d * sc) * acc - (dmin * mn) * aux[g];
+        }
+        return total;
+    }
+    __device__ __forceinline__ static void decode(const uint32_t* r, float* w) {
+        const float d = half_bits_to_float(r[0] & 0xFFFFu), dmin = half_bits_to_float(r[0] >> 16);
+        const uint32_t sc_lo = r[1] & 0x3F3F3F3Fu, mn_lo = r[2] & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (r[3] & 0x0F0F0F0Fu) | ((r[1] >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((r[3] >> 4) & 0x0F0F0F0Fu) | ((r[2] >> 2) & 0x30303030u);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            const float scale = d * ubyte_f(g < 4 ? sc_lo : sc_hi, g & 3);
+            const float floor_ = dmin * ubyte_f(g < 4 ? mn_lo : mn_hi, g & 3);
+#pragma unroll
+            for (int m = 0; m < 2; ++m) {
+                const uint32_t qs = r[4 + 2 * (g >> 1) + m];
+                const uint32_t code = (g & 1) ? ((qs >> 4) & 0x0F0F0F0Fu) : (qs & 0x0F0F0F0Fu);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[8 * g + 4 * m + j] = scale * ubyte_f(code, j) - floor_;
+            }
+        }
+    }
+    __device__ __forceinline__ static int kstep(int u, int m) { return (u >> 2) * 256 + (u & 3) * 8 + 32 * m; }
+};
+
 // ---- BF16 -----------------------------------------------------------------------------------
 template <> struct Unit64<QMOE_FMT_BF16> {
     static constexpr int RAW = 32, AUX = 1;
@@ -342,6 +405,7 @@ __device__ __forceinline__ int64_t row_bytes_dev(int fmt, int k) {
     switch (fmt) {
     case QMOE_FMT_Q8_0: return (int64_t)(k >> 5) * 34;
     case QMOE_FMT_Q5_K: return (int64_t)(k >> 8) * 176;
+    case QMOE_FMT_Q4_K: return (int64_t)(k >> 8) * 144;
     case QMOE_FMT_Q6_K: return (int64_t)(k >> 8) * 210;
     default: return (int64_t)k * 2;
     }

@@ -88,7 +88,7 @@ def test_expert_view_of_a_bank_is_offset_aligned(cuda):
     np.testing.assert_array_equal(bits(view.dequantize().cpu().numpy()), bits(R.dequantize(one.data, one.shape, "Q6_K")))
 
 
-@pytest.mark.parametrize("fmt,shape", [("Q8_0", (4096, 4096)), ("Q6_K", (1024, 4096)), ("Q5_K", (1024, 4096))])
+@pytest.mark.parametrize("fmt,shape", [("Q8_0", (4096, 4096)), ("Q6_K", (1024, 4096)), ("Q5_K", (1024, 4096)), ("Q4_K", (1024, 4096))])
 def test_full_size_matrix_bit_exact(cuda, fmt, shape):
     announce("dequant full size", fmt, shape)
     w = synthetic.packed_weight(fmt, shape, 106)

@@ -71,7 +71,7 @@ def test_large_output_projection_exact(cuda, rows, tokens):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, BF16_MAX_ABS)])
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "Q4_K", "BF16"])
 def test_linear_low_precision_activations(cuda, dtype, tol, fmt):
     announce("linear lowp", fmt, dtype)
     w = synthetic.packed_weight(fmt, (64, 512), 7)
@@ -135,7 +135,7 @@ def test_linear_batch_equals_separate_calls(cuda, tokens):
         assert rel_l2(out.cpu().numpy(), R.linear(xh, *triple(host))) <= 2e-5 <= REL_L2
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "Q4_K", "BF16"])
 @pytest.mark.parametrize("tokens,dtype", [(5, "f32"), (40, "f32"), (17, "f16"), (33, "bf16")])
 def test_linear_batch_token_batches_long_rows(cuda, fmt, tokens, dtype):
     """Token batches through one batched launch: rows of 8192 and 14336 columns (split over the
@@ -160,7 +160,7 @@ def test_linear_batch_token_batches_long_rows(cuda, fmt, tokens, dtype):
             assert np.abs(out.float().cpu().numpy() - want).max() <= tol * scale
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "Q4_K", "BF16"])
 @pytest.mark.parametrize("k", [512, 1024, 2048, 6144, 8192, 14336])
 def test_single_token_streaming_every_row_width(cuda, fmt, k):
     """One token through the streaming kernel at every lane layout: 8 / 16 / 32 lanes per row,
@@ -185,7 +185,7 @@ def test_single_token_streaming_every_row_width(cuda, fmt, k):
     assert rel_l2(h, R.swiglu(x, triple(hosts[0]), triple(hosts[1]))) <= 5e-6 <= REL_L2
 
 
-@pytest.mark.parametrize("gf,uf", [("Q8_0", "Q8_0"), ("Q5_K", "Q4_K"), ("Q6_K", "Q6_K"), ("Q5_K", "Q5_K"), ("BF16", "Q8_0")])
+@pytest.mark.parametrize("gf,uf", [("Q8_0", "Q8_0"), ("Q5_K", "Q4_K"), ("Q6_K", "Q6_K"), ("Q5_K", "Q5_K"), ("Q4_K", "Q4_K"), ("BF16", "Q8_0")])
 @pytest.mark.parametrize("m", [1, 3, 16])
 def test_swiglu_fused_matches_oracle_and_unfused(cuda, gf, uf, m):
     announce("swiglu", gf, uf, m)
@@ -209,7 +209,7 @@ def test_swiglu_fused_matches_oracle_and_unfused(cuda, gf, uf, m):
         quantized_swiglu(xd, dg, object())
 
 
-@pytest.mark.parametrize("fmts", [("Q8_0", "Q8_0", "Q8_0"), ("Q5_K", "Q5_K", "Q6_K"), ("Q6_K", "Q6_K", "Q6_K")])
+@pytest.mark.parametrize("fmts", [("Q8_0", "Q8_0", "Q8_0"), ("Q5_K", "Q5_K", "Q6_K"), ("Q6_K", "Q6_K", "Q6_K"), ("Q4_K", "Q4_K", "Q4_K")])
 @pytest.mark.parametrize("fuse", [True, False])
 def test_packed_expert_matches_oracle(cuda, fmts, fuse):
     announce("expert", fmts, fuse)
@@ -236,7 +236,7 @@ def test_expert_reference_native_vector(cuda):
     np.testing.assert_allclose(got, RV["expert_out"], rtol=3e-5, atol=2e-4 * np.abs(RV["expert_out"]).max())
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "Q4_K", "BF16"])
 @pytest.mark.parametrize("shape", [(4096, 4096), (1024, 4096), (4096, 14336)])
 def test_8b_projection_shapes_linearity_and_row_checks(cuda, fmt, shape):
     """Full-size shapes: spot rows against the oracle plus linearity in x (size-independent)."""

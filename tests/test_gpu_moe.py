@@ -51,7 +51,7 @@ def oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec):
     return R.moe_forward(hidden, logits, k, e, expert_fn, tuple(triple(w) for w in shared), gate_vec)
 
 
-@pytest.mark.parametrize("fmts", [("Q8_0", "Q8_0", "Q8_0"), ("Q6_K", "Q6_K", "Q6_K"), ("Q5_K", "Q5_K", "Q6_K")])
+@pytest.mark.parametrize("fmts", [("Q8_0", "Q8_0", "Q8_0"), ("Q6_K", "Q6_K", "Q6_K"), ("Q5_K", "Q5_K", "Q6_K"), ("Q4_K", "Q4_K", "Q4_K")])
 @pytest.mark.parametrize("tokens", [1, 4, 16, 40])
 def test_moe_step_matches_oracle(cuda, fmts, tokens):
     announce("moe step", fmts, tokens)
@@ -171,7 +171,7 @@ def test_combine_order_is_ascending_expert_id(cuda):
 
 
 # ---- grouped single-token decode (pointer table) ------------------------------------------------
-FORMATS = [("Q8_0", "Q8_0", "Q8_0"), ("Q5_K", "Q4_K", "Q6_K"), ("Q6_K", "Q6_K", "Q6_K")]
+FORMATS = [("Q8_0", "Q8_0", "Q8_0"), ("Q5_K", "Q4_K", "Q6_K"), ("Q6_K", "Q6_K", "Q6_K"), ("Q4_K", "Q4_K", "Q6_K")]
 
 
 def handles(formats, cuda, d=256, f=256, count=3, seed=10600):
@@ -367,6 +367,8 @@ def test_decode_path_with_more_experts_than_the_fused_launch_routes(cuda, tokens
     (8, 1024, 256, 512, 3, "BF16", 4, "bf16"),
     (8, 1024, 256, 512, 3, "Q5_K", 9, "f16"),     # nine tokens: routing kernel + device-side list, fp16 hidden states
     (8, 2048, 512, 0, 4, "Q6_K", 5, "f32"),       # no shared expert
+    (8, 1024, 256, 512, 3, "Q4_K", 2, "f32"),     # Q4_K bank: fused kernel
+    (8, 1024, 256, 512, 3, "Q4_K", 7, "bf16"),    # Q4_K bank: routing kernel + list
 ])
 def test_decode_shapes_lane_layouts_and_types(cuda, e, d, f, fsh, k, fmt, tokens, dtype):
     """Decode-size steps across the lane layouts of the two kernels (row widths of the gate/up
@@ -376,7 +378,7 @@ def test_decode_shapes_lane_layouts_and_types(cuda, e, d, f, fsh, k, fmt, tokens
     gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh if has_shared else 256, (fmt, fmt, fmt), 3100)
     # exact in bf16 and fp32 (fp16 rounds); the synthetic Q5_K scales / minima make outputs large,
     # so those inputs are kept small enough for fp16 outputs
-    hidden = synthetic.activations((tokens, d), 23, "bf16") * np.float32(2.0 if fmt != "Q5_K" else 2.0 ** -6)
+    hidden = synthetic.activations((tokens, d), 23, "bf16") * np.float32(2.0 if fmt not in ("Q5_K", "Q4_K") else 2.0 ** -6)
     tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
     hd = torch.from_numpy(hidden).to(cuda).to(tdt)
     hidden = hd.float().cpu().numpy()
