@@ -39,7 +39,7 @@ enum {
     QMOE_FMT_Q8_0 = 0,
     QMOE_FMT_Q4_0 = 1,
     QMOE_FMT_Q4_K = 2,
-    QMOE_FMT_Q3_K = 3, /* recognised, not implemented: QMOE_EUNSUPPORTED */
+    QMOE_FMT_Q3_K = 3,
     QMOE_FMT_Q5_K = 4,
     QMOE_FMT_Q6_K = 5,
     QMOE_FMT_BF16 = 100

@@ -11,6 +11,7 @@
 //   Q8_0  34 B / 32 el : f16 d | i8 q[32]
 //   Q4_0  18 B / 32 el : f16 d | u8 qs[16]           (low nibbles el 0..15, high 16..31)
 //   Q4_K 144 B /256 el : f16 d | f16 dmin | u8 sc[12] | u8 qs[128]
+//   Q3_K 110 B /256 el : u8 hmask[32] | u8 qs[64] | u8 sc[12] | f16 d
 //   Q5_K 176 B /256 el : f16 d | f16 dmin | u8 sc[12] | u8 qh[32] | u8 qs[128]
 //   Q6_K 210 B /256 el : u8 ql[128] | u8 qh[64] | i8 sc[16] | f16 d
 //   BF16   2 B /  1 el
@@ -163,6 +164,46 @@ template <int QS_BASE, bool HIGH, int BYTES> struct FmtK45 {
 template <> struct Fmt<QMOE_FMT_Q4_K> : FmtK45<16, false, 144> {};
 template <> struct Fmt<QMOE_FMT_Q5_K> : FmtK45<48, true, 176> {};
 
+// Q3_K: a unit is byte quad jj of the 32-byte lanes: one hmask dword and the two qs dwords ->
+// 32 weights, four from each 32-element plane.  w = (d*(sc-32)) * (q2 - 4*(1-hbit))
+// (mini_llm/ops/quantized_weight.py:251-266, native_packed_cpu.cpp:177-193).
+template <> struct Fmt<QMOE_FMT_Q3_K> {
+    static constexpr int BLOCK_ELEMS = 256, BLOCK_BYTES = 110;
+    static constexpr int UNIT = 32, GROUPS = 8;
+    __device__ static int units_per_row(int k) { return k / 32; }
+    __device__ static int xoff(int u, int g) { return (u >> 3) * 256 + 32 * g + 4 * (u & 7); }
+    // six-bit scale of 16-element group g, minus 32
+    __device__ static int scale_of(const uint8_t* sb, int g) {
+        const uint32_t lo = ((uint32_t)sb[g & 7] >> (4 * (g >> 3))) & 15u;
+        const uint32_t hi = ((uint32_t)sb[8 + (g & 3)] >> (2 * (g >> 2))) & 3u;
+        return (int)(lo | (hi << 4)) - 32;
+    }
+    __device__ static void decode(const uint8_t* row, int u, float* w) {
+        const uint8_t* p = row + (size_t)(u >> 3) * 110;
+        const int jj = u & 7;
+        const uint32_t hm = ld_u32_a2(p + 4 * jj);
+        const uint32_t q0 = ld_u32_a2(p + 32 + 4 * jj), q1 = ld_u32_a2(p + 64 + 4 * jj);
+        const float d = half_bits_to_float(ld_u16(p + 108));
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            const float scale = d * (float)scale_of(p + 96, 2 * g + (jj >> 2));
+            const uint32_t qs = g < 4 ? q0 : q1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int low = (int)((qs >> (8 * j + 2 * (g & 3))) & 3u);
+                const int keep = (int)((hm >> (8 * j + g)) & 1u);
+                w[4 * g + j] = scale * (float)(low - 4 * (1 - keep));
+            }
+        }
+    }
+    __device__ static float element(const uint8_t* blk, int i) {
+        const int low = (blk[32 + (i >> 7) * 32 + (i & 31)] >> (2 * ((i & 127) >> 5))) & 3;
+        const int keep = (blk[i & 31] >> (i >> 5)) & 1;
+        const float scale = half_bits_to_float(ld_u16(blk + 108)) * (float)scale_of(blk + 96, i >> 4);
+        return scale * (float)(low - 4 * (1 - keep));
+    }
+};
+
 // Q6_K: a unit is byte quad jj of one 128-element half h: two ql dwords and one qh
 // dword -> 16 weights, four from each 32-element quarter of the half.
 template <> struct Fmt<QMOE_FMT_Q6_K> {
@@ -241,7 +282,7 @@ inline int block_bytes(int fmt) {
     }
 }
 inline bool format_implemented(int fmt) {
-    return fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q4_0 || fmt == QMOE_FMT_Q4_K ||
+    return fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q4_0 || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_Q3_K ||
            fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_BF16;
 }
 inline int64_t row_bytes(int fmt, int64_t k) { return k / block_elems(fmt) * block_bytes(fmt); }

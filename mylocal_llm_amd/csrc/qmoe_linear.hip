@@ -259,6 +259,7 @@ int qmoe_dequantize(const void* w, int fmt, int64_t n, int64_t k, float* out, vo
     switch (fmt) {
     case QMOE_FMT_Q8_0: return launch_dequant<QMOE_FMT_Q8_0>(w, n, k, out, s);
     case QMOE_FMT_Q4_0: return launch_dequant<QMOE_FMT_Q4_0>(w, n, k, out, s);
+    case QMOE_FMT_Q3_K: return launch_dequant<QMOE_FMT_Q3_K>(w, n, k, out, s);
     case QMOE_FMT_Q4_K: return launch_dequant<QMOE_FMT_Q4_K>(w, n, k, out, s);
     case QMOE_FMT_Q5_K: return launch_dequant<QMOE_FMT_Q5_K>(w, n, k, out, s);
     case QMOE_FMT_Q6_K: return launch_dequant<QMOE_FMT_Q6_K>(w, n, k, out, s);

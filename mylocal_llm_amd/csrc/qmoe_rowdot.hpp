@@ -43,6 +43,7 @@ __device__ __forceinline__ void row_dot(int fmt, const uint8_t* __restrict__ row
     switch (fmt) {
     case QMOE_FMT_Q8_0: row_dot_fmt<QMOE_FMT_Q8_0, XDT, MT>(row, k, fast, x, xbase, lane, acc); break;
     case QMOE_FMT_Q4_0: row_dot_fmt<QMOE_FMT_Q4_0, XDT, MT>(row, k, fast, x, xbase, lane, acc); break;
+    case QMOE_FMT_Q3_K: row_dot_fmt<QMOE_FMT_Q3_K, XDT, MT>(row, k, fast, x, xbase, lane, acc); break;
     case QMOE_FMT_Q4_K: row_dot_fmt<QMOE_FMT_Q4_K, XDT, MT>(row, k, fast, x, xbase, lane, acc); break;
     case QMOE_FMT_Q5_K: row_dot_fmt<QMOE_FMT_Q5_K, XDT, MT>(row, k, fast, x, xbase, lane, acc); break;
     case QMOE_FMT_Q6_K: row_dot_fmt<QMOE_FMT_Q6_K, XDT, MT>(row, k, fast, x, xbase, lane, acc); break;

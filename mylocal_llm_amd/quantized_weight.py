@@ -22,6 +22,7 @@ BLOCK_FORMATS = {
     "Q8_0": (32, 34),
     "Q4_0": (32, 18),
     "Q4_K": (256, 144),
+    "Q3_K": (256, 110),
     "Q5_K": (256, 176),
     "Q6_K": (256, 210),
     "BF16": (1, 2),

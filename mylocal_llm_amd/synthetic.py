@@ -6,6 +6,7 @@ Block contents follow the workload descriptions of the benchmark configurations:
         U[-64, 63], fp16 super-scale |N(5e-4, 1e-4)|
   Q5_K  5-bit codes uniform in [0, 31], eight 6-bit (scale, min) pairs U[0, 63], fp16 d and dmin
   Q4_K  as Q5_K without the high-bit plane;  Q4_0  nibbles uniform, fp16 d
+  Q3_K  mask, 2-bit codes and 6-bit scales uniform, fp16 d
   BF16  N(0, 0.02) rounded to nearest-even bf16
 All generators return a flat uint8 array in GGUF block layout for shape [..., K].
 """
@@ -45,6 +46,9 @@ def pack_blocks(fmt, rng, nblocks):
         blk[:, 2:4] = _scale(rng, nblocks)
         blk[:, 4:16] = _pack_scale_min(rng.integers(0, 64, (nblocks, 8)), rng.integers(0, 64, (nblocks, 8)))
         blk[:, 16:] = rng.integers(0, 256, (nblocks, nbytes - 16), dtype=np.uint8)
+    elif fmt == "Q3_K":
+        blk[:, 0:108] = rng.integers(0, 256, (nblocks, 108), dtype=np.uint8)
+        blk[:, 108:110] = _scale(rng, nblocks)
     elif fmt == "Q6_K":
         blk[:, 0:192] = rng.integers(0, 256, (nblocks, 192), dtype=np.uint8)
         blk[:, 192:208] = rng.integers(-64, 64, (nblocks, 16)).astype(np.int8).view(np.uint8)

@@ -12,6 +12,7 @@
  *   Q8_0  w = d*q                    mini_llm/ops/quantized_weight.py:208-211
  *   Q4_0  w = d*(nibble-8)           mini_llm/ops/quantized_weight.py:212-216
  *   Q4_K/Q5_K w=(d*sc)*q - dmin*mn   mini_llm/ops/quantized_weight.py:217-237
+ *   Q3_K  w = (d*(sc-32))*(q2-4*(1-h)) mini_llm/ops/quantized_weight.py:251-266
  *   Q6_K  w = (d*sc)*q               mini_llm/ops/quantized_weight.py:238-250
  *   BF16  bits<<16                   mini_llm/external/gguf_tensor.py:48-51
  *   host linear x @ W.T (fp32)       mini_llm/ops/quantized_linear.py:303-305
@@ -30,7 +31,7 @@ enum { F_Q8_0 = 0, F_Q4_0 = 1, F_Q4_K = 2, F_Q3_K = 3, F_Q5_K = 4, F_Q6_K = 5, F
 static int fmt_elems(int f) {
     switch (f) {
     case F_Q8_0: case F_Q4_0: return 32;
-    case F_Q4_K: case F_Q5_K: case F_Q6_K: return 256;
+    case F_Q4_K: case F_Q5_K: case F_Q6_K: case F_Q3_K: return 256;
     case F_BF16: return 1;
     default: return 0;
     }
@@ -40,6 +41,7 @@ static int fmt_bytes(int f) {
     case F_Q8_0: return 34;
     case F_Q4_0: return 18;
     case F_Q4_K: return 144;
+    case F_Q3_K: return 110;
     case F_Q5_K: return 176;
     case F_Q6_K: return 210;
     case F_BF16: return 2;
@@ -86,6 +88,14 @@ static float decode_element(int fmt, const uint8_t* b, int i) {
         float scale = half_at(b) * (float)sc;
         float floor_ = half_at(b + 2) * (float)mn;
         return scale * (float)q - floor_;
+    }
+    if (fmt == F_Q3_K) { /* mini_llm/ops/native_packed_cpu.cpp:177-193, one element at a time */
+        int g = i / 16;
+        int sc = (int)(((b[96 + g % 8] >> (4 * (g / 8))) & 15) | (((b[104 + g % 4] >> (2 * (g / 4))) & 3) << 4)) - 32;
+        int two = (b[32 + (i / 128) * 32 + i % 32] >> (2 * ((i % 128) / 32))) & 3;
+        int keep = (b[i % 32] >> (i / 32)) & 1;
+        float scale = half_at(b + 108) * (float)sc;
+        return scale * (float)(two - 4 * (1 - keep));
     }
     if (fmt == F_Q6_K) {
         int h = i / 128, r = i % 128;

@@ -36,6 +36,7 @@ BLOCKS = {
     "Q8_0": (32, 34),
     "Q4_0": (32, 18),
     "Q4_K": (256, 144),
+    "Q3_K": (256, 110),
     "Q5_K": (256, 176),
     "Q6_K": (256, 210),
     "BF16": (1, 2),
@@ -87,7 +88,7 @@ def dequantize(data, shape, fmt):
     Restates PackedGGUFWeight.dequantize_reference (quantized_weight.py:151-250)
     for the formats on the path.  The float operation order of the reference is
     kept -- ``d*q`` (Q8_0 :208-211), ``(d*sc)*q - dmin*mn`` (Q4_K/Q5_K :217-237),
-    ``(d*sc)*q`` (Q6_K :238-250) -- so the result is bit-identical, signed zeros
+    ``(d*sc)*q`` (Q6_K :238-250, Q3_K :251-266) -- so the result is bit-identical, signed zeros
     included.
     """
     if fmt == "BF16":
@@ -123,6 +124,22 @@ def dequantize(data, shape, fmt):
             scale = d * sc[:, g].astype(np.float32)
             floor = dmin * mn[:, g].astype(np.float32)
             out[:, 32 * g:32 * g + 32] = scale[:, None] * q.astype(np.float32) - floor[:, None]
+    elif fmt == "Q3_K":
+        # quantized_weight.py:251-266: 2 low bits in qs, a "keep" bit in hmask (0 -> minus four),
+        # sixteen 6-bit scales minus 32; w = (d * scale) * value.
+        d = _half_field(blk, 108)
+        sb = blk[:, 96:108]
+        for g in range(16):
+            low = (sb[:, g % 8] >> (4 * (g // 8))) & 15
+            high = (sb[:, 8 + g % 4] >> (2 * (g // 4))) & 3
+            scale = d * ((low | (high << 4)).astype(np.float32) - np.float32(32))
+            first = 16 * g  # elements first..first+15: plane i // 32, byte lane i % 32
+            lanes = np.arange(first, first + 16) % 32
+            plane = first // 32
+            two = (blk[:, 32 + (first // 128) * 32 + lanes] >> (2 * (plane % 4))) & 3
+            keep = (blk[:, lanes] >> plane) & 1
+            value = two.astype(np.int32) - 4 * (1 - keep.astype(np.int32))
+            out[:, first:first + 16] = scale[:, None] * value.astype(np.float32)
     elif fmt == "Q6_K":
         d = _half_field(blk, 208)
         sub = np.ascontiguousarray(blk[:, 192:208]).view(np.int8).astype(np.float32)
@@ -338,6 +355,7 @@ PINNING = {
     "dequantize/Q8_0": "closed form d*int8; large-output vector of tests/test_0106p (q=(row%15-7), d=.125)",
     "dequantize/Q4_0": "hand-packed vector of tests/test_0106a:18-25",
     "dequantize/Q4_K": "hand-packed vector of tests/test_0106a:28-33",
+    "dequantize/Q3_K": "hand-packed mask / scale vectors of tests/test_0106a:36-43 (+2 / -2) + independent per-element scalar decode (oracle.c) + oracle/_ref where it builds",
     "dequantize/Q5_K": "hand-packed vectors of tests/test_0106g:23-45 (8.25 / 9.0) + independent per-lane scalar decode",
     "dequantize/Q6_K": "all-codes signed-extremes vector of tests/test_0106l_q6k:25-46 + independent per-lane scalar decode",
     "bf16_expand": "all 65536 patterns == word<<16 and the byte fixture of tests/test_0106l_gguf_bf16:47-57",

@@ -4,6 +4,7 @@ The cases are the known-answer vectors held by the reference's own tests, re-enc
 as data (packed bytes in, fp32 values out):
   q4_0_nibbles      tests/test_0106a_packed_gguf.py:18-25   d=.5, every byte 0x83
   q4_k_scales       tests/test_0106a_packed_gguf.py:28-33   d=1, dmin=0, four groups scale 1
+  q3_k_keep / q3_k_minus4  tests/test_0106a_packed_gguf.py:36-43   every scale 33-32=1, every code 2, mask all ones / all zeros
   q5_k_group0       tests/test_0106g_q5k_packed.py:23-35    8.25 x32 then zeros
   q5_k_group7       tests/test_0106g_q5k_packed.py:37-45    zeros then 9.0 x32
   q6_k_all_codes    tests/test_0106l_q6k_packed.py:25-46    every 6-bit code x 16 signed scales
@@ -30,6 +31,12 @@ def main():
     out["q4_k_scales_blocks"] = np.concatenate(
         [f16(1), f16(0), np.array([1] * 4 + [0] * 8, np.uint8), np.full(128, 0x12, np.uint8)])
     out["q4_k_scales_expected"] = np.array(([2.0] * 32 + [1.0] * 32) * 2 + [0.0] * 128, np.float32)
+    # Q3_K: scale bytes 0x11 x8 + 0xAA x4 -> every six-bit scale 33 (= +1), qs 0xAA -> every code 2;
+    # mask bit 1 keeps the code, 0 subtracts four
+    for name, mask, value in (("q3_k_keep", 0xFF, 2.0), ("q3_k_minus4", 0x00, -2.0)):
+        out[name + "_blocks"] = np.concatenate([np.full(32, mask, np.uint8), np.full(64, 0xAA, np.uint8),
+                                                np.array([0x11] * 8 + [0xAA] * 4, np.uint8), f16(1)])
+        out[name + "_expected"] = np.full(256, value, np.float32)
     # Q5_K group 0: d=.5 dmin=.25 scale0=1 min0=1, high bit of group 0 set, nibbles 0x21
     raw = np.zeros(176, np.uint8)
     raw[0:2], raw[2:4] = f16(0.5), f16(0.25)

@@ -5,6 +5,7 @@ oracle/_ref/) on small seeded inputs:
                                i.e. every decoded coefficient as the reference decodes it
   <fmt>_x / <fmt>_gemv         random activations and the reference's GEMV result
   expert_*                     one Q5_K/Q5_K/Q6_K SwiGLU expert through mylocal_packed_expert
+  (formats: Q8_0, Q4_0, Q4_K, Q5_K, Q6_K, Q3_K)
 Only this container has the reference checkout; the vectors travel, the reference does not.
 Run from the repository root after `make -C oracle`: python tests/golden/make_ref_vectors.py
 """
@@ -52,6 +53,19 @@ def main():
     x = rng.standard_normal((2, d), dtype=np.float32) * 0.5
     out["expert_gate"], out["expert_up"], out["expert_down"], out["expert_x"] = gate, up, down, x
     out["expert_out"] = native.ref_expert(x, (gate, (f, d), "Q5_K"), (up, (f, d), "Q5_K"), (down, (d, f), "Q6_K"))
+    # Q3_K, from a generator of its own so that the vectors above stay as they were
+    rng3 = np.random.default_rng(20253)
+    rows, k = 6, 512
+    nblocks = rows * k // 256
+    blk = rng3.integers(0, 256, (nblocks, 110), dtype=np.uint8)
+    s = rng3.normal(0, 0.01, nblocks).astype("<f2")
+    s[0] = np.float16(3e-6)
+    blk[:, 108:110] = s.view(np.uint8).reshape(nblocks, 2)
+    x = rng3.standard_normal((3, k), dtype=np.float32)
+    out["Q3_K_blocks"] = blk
+    out["Q3_K_dense"] = native.ref_gemv(np.eye(k, dtype=np.float32), blk, (rows, k), "Q3_K").T.copy()
+    out["Q3_K_x"] = x
+    out["Q3_K_gemv"] = native.ref_gemv(x, blk, (rows, k), "Q3_K")
     np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "ref_native_vectors.npz"), **out)
 
 

@@ -14,14 +14,14 @@ pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FV = np.load(os.path.join(GOLDEN, "format_vectors.npz"))
 RV = np.load(os.path.join(GOLDEN, "ref_native_vectors.npz"))
-FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K", "BF16"]
+FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K", "BF16"]
 
 
 def bits(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
 
 
-@pytest.mark.parametrize("case,fmt", [("q4_0_nibbles", "Q4_0"), ("q4_k_scales", "Q4_K"),
+@pytest.mark.parametrize("case,fmt", [("q4_0_nibbles", "Q4_0"), ("q4_k_scales", "Q4_K"), ("q3_k_keep", "Q3_K"), ("q3_k_minus4", "Q3_K"),
                                       ("q5_k_group0", "Q5_K"), ("q5_k_group7", "Q5_K"),
                                       ("q6_k_all_codes", "Q6_K")])
 def test_hand_packed_known_answers(cuda, case, fmt):
@@ -32,7 +32,7 @@ def test_hand_packed_known_answers(cuda, case, fmt):
     np.testing.assert_array_equal(got.ravel(), expected)
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K"])
 def test_reference_native_decoder_vectors(cuda, fmt):
     announce("dequant ref vectors", fmt)
     dense = RV[fmt + "_dense"]

@@ -16,7 +16,7 @@ from gpu_util import BF16_MAX_ABS, REL_L2, announce, rel_l2, triple, upload
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 RV = np.load(os.path.join(GOLDEN, "ref_native_vectors.npz"))
-FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K", "BF16"]
+FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K", "BF16"]
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
@@ -45,7 +45,7 @@ def test_config0_single_q8_0_matrix_batch1(cuda):
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K"])
 def test_linear_reference_native_vectors(cuda, fmt):
     blocks, x, y = RV[fmt + "_blocks"], RV[fmt + "_x"], RV[fmt + "_gemv"]
     w = PackedGGUFWeight(blocks, (y.shape[1], x.shape[1]), fmt)

@@ -96,7 +96,7 @@ def test_invalid_arguments_return_codes_before_any_launch():
     assert lib.qmoe_linear(fake, 0, 4, 33, fake, 0, 1, fake, 0, null) == 1      # K not a block multiple
     assert b"multiple" in lib.qmoe_last_error()
     assert lib.qmoe_linear(fake, 0, 4, 32, fake, 0, 0, fake, 0, null) == 1      # no tokens
-    assert lib.qmoe_linear(fake, 3, 4, 256, fake, 0, 1, fake, 0, null) == 2     # Q3_K: recognised, no kernel
+    assert lib.qmoe_linear(fake, 3, 4, 384, fake, 0, 1, fake, 0, null) == 1     # Q3_K: K not a multiple of 256
     assert lib.qmoe_linear(fake, 42, 4, 256, fake, 0, 1, fake, 0, null) == 1    # unknown format
     assert lib.qmoe_linear(fake, 0, 4, 32, fake, 9, 1, fake, 0, null) == 1      # unknown dtype
     assert lib.qmoe_dequantize(fake, 5, 2, 100, fake, null) == 1

@@ -12,10 +12,10 @@ from mylocal_llm_amd import synthetic
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FV = np.load(os.path.join(GOLDEN, "format_vectors.npz"))
 RV = np.load(os.path.join(GOLDEN, "ref_native_vectors.npz"))
-PACKED = ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"]
+PACKED = ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K"]
 
 
-@pytest.mark.parametrize("case,fmt", [("q4_0_nibbles", "Q4_0"), ("q4_k_scales", "Q4_K"),
+@pytest.mark.parametrize("case,fmt", [("q4_0_nibbles", "Q4_0"), ("q4_k_scales", "Q4_K"), ("q3_k_keep", "Q3_K"), ("q3_k_minus4", "Q3_K"),
                                       ("q5_k_group0", "Q5_K"), ("q5_k_group7", "Q5_K"),
                                       ("q6_k_all_codes", "Q6_K")])
 @pytest.mark.parametrize("impl", ["numpy", "c"])

@@ -18,7 +18,7 @@ def triple(w):
     return (w.data, w.shape, w.quant_type)
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q5_K", "Q6_K", "Q4_K", "Q4_0", "BF16"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q5_K", "Q6_K", "Q4_K", "Q3_K", "Q4_0", "BF16"])
 @pytest.mark.parametrize("shape", [(3, 512), (2, 3, 512)])
 def test_linear_is_fp32_matmul_of_dequantised_matrix(fmt, shape):
     w = synthetic.packed_weight(fmt, (7, 512), 11)
@@ -54,7 +54,7 @@ def test_linear_preserves_dtype_and_rejects_bad_shapes(dtype):
         R.linear(np.zeros(64, dtype), *triple(w))
 
 
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K"])
 def test_linear_matches_reference_native_gemv_vectors(fmt):
     blocks, x, y = RV[fmt + "_blocks"], RV[fmt + "_x"], RV[fmt + "_gemv"]
     shape = (y.shape[1], x.shape[1])
