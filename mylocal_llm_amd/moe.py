@@ -10,13 +10,14 @@ combine; expert ids never travel to the host.
 """
 import ctypes
 import math
+from dataclasses import dataclass
 
 import numpy as np
 import torch
 
 from . import _lib
 from .quantized_linear import (
-    DevicePackedGGUFWeight, _FORMAT_ID, _TORCH_DTYPE_ID, _ptr, _stream,
+    DevicePackedGGUFWeight, _FORMAT_ID, _TORCH_DTYPE_ID, _ptr, _stream, _upload_bytes, packed_to_device,
 )
 from .quantized_weight import BLOCK_FORMATS, PackedGGUFWeight
 from .router import RouterInference
@@ -77,7 +78,7 @@ class DevicePackedExpertBank:
             if not torch.cuda.is_available():
                 raise RuntimeError("Packed GPU weights require a HIP device")
             dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
-            return torch.from_numpy(np.ascontiguousarray(item.data)).to(dev), item.shape, item.quant_type
+            return _upload_bytes(item.data, dev), item.shape, item.quant_type
         data, shape, fmt = item
         shape = tuple(int(s) for s in shape)
         if fmt not in BLOCK_FORMATS:
@@ -228,21 +229,124 @@ class ExpertsInference:
         return y.reshape(batch_size, seq_len, d_model)
 
 
+@dataclass(frozen=True)
+class Qwen3NextMoESpec:
+    """Sizes of one Qwen3-Next MoE block, validated against the checkpoint's headers
+    (mini_llm/external/qwen3next_moe.py:21-90); no payload is touched."""
+    d_model: int
+    d_ff: int
+    shared_d_ff: int
+    n_experts: int
+    top_k: int
+
+    @classmethod
+    def from_index(cls, index, layer_id):
+        from .qwen3next_gguf import _DENSE_TYPES, _GGUF_BLOCK_FORMATS, _SHARED, _meta, _positive_integer, _shape
+        if index.architecture not in ('qwen3next', 'qwen3_next'):
+            raise ValueError('Expected Qwen3-Next architecture')
+        if isinstance(layer_id, bool) or not isinstance(layer_id, int):
+            raise TypeError('layer_id must be an integer')
+        if not 0 <= layer_id < index.layers:
+            raise IndexError(f'Invalid Qwen3-Next layer {layer_id}')
+        prefix = index.architecture
+        # pruned / grouped / bias-corrected routing variants are not guessed at
+        for suffix in ('expert_weights_scale', 'expert_weights_norm', 'expert_gating_func',
+                       'expert_group_count', 'expert_group_used_count'):
+            if f'{prefix}.{suffix}' in index.reader.fields:
+                raise NotImplementedError(f'Unsupported explicit routing metadata {suffix}')
+        spec = cls(
+            _positive_integer(index.d_model, 'd_model'),
+            _positive_integer(index.d_ff, 'd_ff'),
+            _positive_integer(_meta(index.reader, f'{prefix}.expert_shared_feed_forward_length'),
+                              'expert_shared_feed_forward_length'),
+            _positive_integer(index.expert_count, 'expert_count'),
+            _positive_integer(index.experts_per_token, 'expert_used_count'),
+        )
+        explicit_ff = _meta(index.reader, f'{prefix}.expert_feed_forward_length', spec.d_ff)
+        if _positive_integer(explicit_ff, 'expert_feed_forward_length') != spec.d_ff:
+            raise ValueError('Expert width metadata disagrees with routed tensors')
+        if spec.top_k > spec.n_experts:
+            raise ValueError('expert_used_count exceeds expert_count')
+        stem = f'blk.{layer_id}.'
+        shapes = {
+            'ffn_gate_inp.weight': (spec.n_experts, spec.d_model),
+            'ffn_gate_inp_shexp.weight': (spec.d_model,),
+            'ffn_gate_shexp.weight': (spec.shared_d_ff, spec.d_model),
+            'ffn_up_shexp.weight': (spec.shared_d_ff, spec.d_model),
+            'ffn_down_shexp.weight': (spec.d_model, spec.shared_d_ff),
+            'ffn_down_exps.weight': (spec.n_experts, spec.d_model, spec.d_ff),
+        }
+        if stem + 'ffn_gate_up_exps.weight' in index.tensors:
+            shapes['ffn_gate_up_exps.weight'] = (spec.n_experts, 2 * spec.d_ff, spec.d_model)
+        else:
+            shapes['ffn_gate_exps.weight'] = (spec.n_experts, spec.d_ff, spec.d_model)
+            shapes['ffn_up_exps.weight'] = (spec.n_experts, spec.d_ff, spec.d_model)
+        for name in index.tensors:
+            if name.startswith(stem + 'ffn_') and name[len(stem):] not in shapes:
+                raise NotImplementedError(f'Unsupported FFN tensor/layout {name}')
+        for suffix, shape in shapes.items():
+            tensor = index.tensors.get(stem + suffix)
+            if tensor is None:
+                raise ValueError(f'Missing MoE tensor {stem + suffix}')
+            if _shape(tensor) != shape:
+                raise ValueError(f'{stem + suffix}: expected shape {shape}, got {_shape(tensor)}')
+            kind = tensor.tensor_type.name
+            allowed = (set(_GGUF_BLOCK_FORMATS) if '_exps.weight' in suffix else
+                       _DENSE_TYPES | set(_GGUF_BLOCK_FORMATS) if suffix in _SHARED else _DENSE_TYPES)
+            if kind not in allowed:
+                raise NotImplementedError(f'{stem + suffix}: unsupported GGUF type {kind}')
+            if kind in _GGUF_BLOCK_FORMATS and shape[-1] % _GGUF_BLOCK_FORMATS[kind][0]:
+                raise ValueError(f'{stem + suffix}: innermost dimension must be block-aligned')
+        return spec
+
+
 class Qwen3NextMoEInference:
     """Renormalised routed SwiGLU experts plus a sigmoid-gated shared SwiGLU expert."""
 
     def __init__(self, bank, top_k, router_weight, shared, shared_gate, *, normalization_floor=2.0 ** -14):
         """router_weight: fp32 [E, D] (GGUF ffn_gate_inp orientation); shared: (gate, up, down)
-        DevicePackedGGUFWeight triple; shared_gate: fp32 [D]."""
+        DevicePackedGGUFWeight triple, or three dense fp32 [out, in] tensors (checkpoints that keep
+        the shared expert in F32 / F16); shared_gate: fp32 [D]."""
         self.bank = bank
         self.top_k = int(top_k)
         self.router = RouterInference(bank.d_model, bank.n_experts, self.top_k,
                                       renormalize_selected=True, normalization_floor=normalization_floor)
         self.router.W_router = router_weight.to(torch.float32).t().contiguous()
         self.router.b_router = torch.zeros(bank.n_experts, dtype=torch.float32, device=router_weight.device)
-        self.shared = shared
+        self.shared_is_dense = all(isinstance(w, torch.Tensor) for w in shared)
+        if not self.shared_is_dense and not all(isinstance(w, DevicePackedGGUFWeight) for w in shared):
+            raise TypeError('shared expert: three DevicePackedGGUFWeight or three dense tensors')
+        self.shared = tuple(w.to(torch.float32).contiguous() for w in shared) if self.shared_is_dense else shared
         self.shared_gate = shared_gate.to(torch.float32).contiguous()
         self.experts = ExpertsInference(bank.d_model, bank.d_ff, bank.n_experts, expert_executor=bank)
+
+    @classmethod
+    def from_index(cls, index, layer_id, *, expert_executor=None, device=None):
+        """Build the block of ``layer_id`` from a ``Qwen3NextGGUFIndex``
+        (mini_llm/external/qwen3next_moe.py:100-127).  ``expert_executor`` may be a resident
+        ``DevicePackedExpertBank`` the caller already holds for this layer; otherwise the
+        layer's routed tensors are uploaded."""
+        spec = Qwen3NextMoESpec.from_index(index, layer_id)
+        if not torch.cuda.is_available():
+            raise RuntimeError('Packed GPU weights require a HIP device')
+        dev = torch.device('cuda', torch.cuda.current_device()) if device is None else torch.device(device)
+        bank = expert_executor if expert_executor is not None else index.expert_bank(layer_id, dev)
+        if (bank.d_model, bank.d_ff) != (spec.d_model, spec.d_ff) or bank.n_experts != spec.n_experts:
+            raise ValueError('Executor dimensions do not match MoE tensors')
+        stem = f'blk.{layer_id}.'
+
+        def dense(name):
+            return torch.from_numpy(np.ascontiguousarray(index.non_expert_weight(stem + name), dtype=np.float32)).to(dev)
+
+        host = [index.projection(stem + name) for name in ('ffn_gate_shexp.weight', 'ffn_up_shexp.weight', 'ffn_down_shexp.weight')]
+        if all(isinstance(w, PackedGGUFWeight) for w in host):
+            shared = tuple(packed_to_device(w, dev) for w in host)
+        else:  # any F32 / F16 projection: the shared expert runs as dense fp32 matmuls
+            shared = tuple(torch.from_numpy(np.ascontiguousarray(
+                w.dequantize_reference() if isinstance(w, PackedGGUFWeight) else w, dtype=np.float32)).to(dev) for w in host)
+        result = cls(bank, spec.top_k, dense('ffn_gate_inp.weight'), shared, dense('ffn_gate_inp_shexp.weight'))
+        result.index, result.layer_id, result.spec = index, layer_id, spec
+        return result
 
     def forward(self, hidden):
         if not isinstance(hidden, torch.Tensor) or hidden.dtype != torch.float32:
@@ -254,6 +358,16 @@ class Qwen3NextMoEInference:
         b, t, d = hidden.shape
         flat = hidden.reshape(b * t, d).contiguous()
         logits = (flat @ self.router.W_router + self.router.b_router).contiguous()
-        out = moe_step(flat, self.bank, self.top_k, logits=logits, shared=self.shared,
-                       shared_gate=self.shared_gate, floor=self.router.normalization_floor)
+        if self.shared_is_dense:
+            # routed part on the packed kernels; shared expert and its admission gate as fp32
+            # matmuls (mini_llm/external/gguf_projection.py:40-88, qwen3next_moe.py:145-147)
+            routed = moe_step(flat, self.bank, self.top_k, logits=logits, floor=self.router.normalization_floor)
+            gate_w, up_w, down_w = self.shared
+            g = flat @ gate_w.t()
+            act = (g * (1.0 / (1.0 + torch.exp(-g)))) * (flat @ up_w.t())
+            sig = torch.exp(-torch.logaddexp(torch.zeros((), device=flat.device), -(flat @ self.shared_gate)))
+            out = routed + (act @ down_w.t()) * sig[:, None]
+        else:
+            out = moe_step(flat, self.bank, self.top_k, logits=logits, shared=self.shared,
+                           shared_gate=self.shared_gate, floor=self.router.normalization_floor)
         return out.reshape(b, t, d)

@@ -75,6 +75,16 @@ class DevicePackedGGUFWeight:
         return out
 
 
+def _upload_bytes(array, device):
+    """uint8 bytes (possibly a read-only view of a memory-mapped file) as a tensor on ``device``."""
+    import warnings
+    array = np.ascontiguousarray(array)
+    with warnings.catch_warnings():
+        # the host tensor is only the source of the copy and is never written through
+        warnings.filterwarnings("ignore", message="The given NumPy array is not writable")
+        return torch.from_numpy(array).to(device)
+
+
 def packed_to_device(weight, device=None):
     """Upload the *packed bytes* of one matrix/expert to HBM once (no expansion)."""
     if not isinstance(weight, PackedGGUFWeight) or len(weight.shape) != 2:
@@ -85,8 +95,7 @@ def packed_to_device(weight, device=None):
         raise RuntimeError("Packed GPU weights require a HIP device")
     _lib.load()
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
-    data = torch.from_numpy(np.ascontiguousarray(weight.data)).to(device)
-    return DevicePackedGGUFWeight(data, weight.shape, weight.quant_type)
+    return DevicePackedGGUFWeight(_upload_bytes(weight.data, device), weight.shape, weight.quant_type)
 
 
 def _check_activation(x, what):
