@@ -155,8 +155,11 @@ def cpu_baseline(budget_s=12.0):
             "numpy": np.__version__, "host_cpus": os.cpu_count()}
 
 
-def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup):
-    """512-expert top-10 MoE decode step (D=2048, F=512, shared F=2048) over rotating banks."""
+def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=False):
+    """512-expert top-10 MoE decode step (D=2048, F=512, shared F=2048) over rotating banks.
+    With ``layer_half`` a step is the second half of a decoder layer: RMSNorm + router logits of the
+    fp32 residual stream in one launch, the MoE step on the normalised rows, residual added in its
+    last kernel (fp32 in, fp32 out)."""
     from mylocal_llm_amd import _lib
     from mylocal_llm_amd.moe import DevicePackedExpertBank, moe_step
     from mylocal_llm_amd.quantized_linear import DevicePackedGGUFWeight
@@ -172,31 +175,44 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup):
         banks.append(DevicePackedExpertBank((g, (e, f, d), fmt), (u, (e, f, d), fmt), (dn, (e, d, f), fmt)))
         shareds.append(tuple(DevicePackedGGUFWeight(device_blocks(torch, fmt, n, kk, gen, device), (n, kk), fmt)
                              for n, kk in ((fsh, d), (fsh, d), (d, fsh))))
-    hidden = torch.randn((tokens, d), device=device, generator=gen).to(torch.bfloat16)
+    hidden = torch.randn((tokens, d), device=device, generator=gen).to(torch.float32 if layer_half else torch.bfloat16)
     logits = torch.randn((n_banks, tokens, e), device=device, generator=gen)
     gate_vec = torch.randn(d, device=device, generator=gen) * 0.02
-    out = torch.empty((tokens, d), device=device, dtype=torch.bfloat16)
+    out = torch.empty((tokens, d), device=device, dtype=hidden.dtype)
+    hdt = 0 if layer_half else 2
+    if layer_half:
+        residual = torch.randn((tokens, d), device=device, generator=gen)
+        gamma = 1 + 0.1 * torch.randn(d, device=device, generator=gen)
+        router_w = torch.randn((n_banks, e, d), device=device, generator=gen) * 0.05
     nbytes_ws = lib.qmoe_moe_workspace_bytes(tokens, k, e, d, f, fsh)
     workspace = torch.empty(nbytes_ws, dtype=torch.uint8, device=device)
     # the C ABI is the boundary: argument structs are built once, a step is one call
     calls = []
     for i in range(n_banks):
         a = _lib.MoeArgs()
-        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), 2, tokens, k
+        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), hdt, tokens, k
         a.logits, a.floor_value, a.renormalize = logits[i].data_ptr(), 2.0 ** -14, 1
+        if layer_half:
+            a.residual = residual.data_ptr()
         banks[i].fill(a.bank)
         g, u, dn = shareds[i]
         a.shared_gate_w, a.shared_up_w, a.shared_down_w = g.data.data_ptr(), u.data.data_ptr(), dn.data.data_ptr()
         a.shared_gate_fmt = a.shared_up_fmt = a.shared_down_fmt = _lib.FORMAT_ID[fmt]
         a.d_ff_shared, a.shared_gate = fsh, gate_vec.data_ptr()
-        a.out, a.out_dtype = out.data_ptr(), 2
+        a.out, a.out_dtype = out.data_ptr(), hdt
         calls.append(a)
     state = {"i": 0}
     wsp = ctypes.c_void_p(workspace.data_ptr())
 
     def fn(stream):
-        a = calls[state["i"] % n_banks]
+        i = state["i"] % n_banks
+        a = calls[i]
         state["i"] += 1
+        if layer_half:  # normalised rows -> `hidden`, logits -> this bank's logits buffer
+            rc = lib.qmoe_norm_router(residual.data_ptr(), tokens, d, gamma.data_ptr(), 1e-6, router_w[i].data_ptr(), None, e,
+                                      hidden.data_ptr(), logits[i].data_ptr(), stream)
+            if rc:
+                raise RuntimeError(lib.qmoe_last_error().decode())
         rc = lib.qmoe_moe_forward(ctypes.byref(a), wsp, nbytes_ws, stream)
         if rc:
             raise RuntimeError(lib.qmoe_last_error().decode())
@@ -207,9 +223,9 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup):
     distinct = sum(len(torch.unique(ids[i])) for i in range(n_banks)) / n_banks
     eb = 3 * weight_bytes(fmt, f, d)
     sb = 3 * weight_bytes(fmt, fsh, d)
-    nbytes = distinct * eb + sb
+    nbytes = distinct * eb + sb + (e * d * 4 if layer_half else 0)
     per_step = ms / steps * 1e-3
-    return {"workload": f"moe_decode_{fmt}_T{tokens}", "ms_per_step": round(ms / steps, 4),
+    return {"workload": f"moe_{'layer_half' if layer_half else 'decode'}_{fmt}_T{tokens}", "ms_per_step": round(ms / steps, 4),
             "weight_bytes": int(nbytes), "distinct_experts": distinct,
             "GBps": round(nbytes / per_step / 1e9, 1), "frac_hbm_peak": round(nbytes / per_step / 1e9 / HBM_PEAK_GBS, 4),
             "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
@@ -244,8 +260,10 @@ def moe_prefill_extra(torch, lib, device, fmt, tokens, steps, warmup):
     calls = []
     for i in range(n_banks):
         a = _lib.MoeArgs()
-        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), 2, tokens, k
+        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), hdt, tokens, k
         a.logits, a.floor_value, a.renormalize = logits[i].data_ptr(), 2.0 ** -14, 1
+        if layer_half:
+            a.residual = residual.data_ptr()
         banks[i].fill(a.bank)
         g, u, dn = shareds[i]
         a.shared_gate_w, a.shared_up_w, a.shared_down_w = g.data.data_ptr(), u.data.data_ptr(), dn.data.data_ptr()
@@ -287,7 +305,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--only", choices=["moe_prefill", "moe_decode"], default=None,
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_layer_half"], default=None,
                     help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device tensor copy (a kernel of known traffic, "
@@ -311,6 +329,9 @@ def main():
         return
     if args.only == "moe_decode":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup) for t in (1, 4, 16)]))
+        return
+    if args.only == "moe_layer_half":
+        print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, layer_half=True) for t in (1, 4)]))
         return
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
@@ -363,6 +384,9 @@ def main():
             torch.cuda.empty_cache()
         for fmt, tokens in (("Q8_0", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q6_K", 1)):
             extras.append(moe_decode_extra(torch, lib, device, fmt, tokens, max(8, args.steps), 3))
+            torch.cuda.empty_cache()
+        for tokens in (1, 4):
+            extras.append(moe_decode_extra(torch, lib, device, "Q8_0", tokens, max(8, args.steps), 3, layer_half=True))
             torch.cuda.empty_cache()
         extras.append(moe_prefill_extra(torch, lib, device, "Q8_0", 512, 6, 2))
         torch.cuda.empty_cache()

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define QMOE_ABI_VERSION 1
+#define QMOE_ABI_VERSION 2
 
 /* Packed formats.  Ids 0..5 are the reference's (_FORMAT_ID,
  * mini_llm/ops/quantized_linear.py:34 and native_packed_cpu.cpp:12).  BF16 has no
@@ -169,6 +169,9 @@ typedef struct qmoe_moe_args {
     int out_dtype;
     float* out_weights;     /* optional [T, k] fp32: routing weights used */
     int64_t* out_ids;       /* optional [T, k] int64: selected experts */
+    /* optional fp32 [T, d_model]: out = residual + (routed + shared * sigmoid), the residual add
+     * that follows the block (mini_llm/external/qwen3next_decoder.py:120) */
+    const float* residual;
 } qmoe_moe_args;
 
 /* Bytes of workspace qmoe_moe_forward needs for these sizes (256-byte aligned). */
@@ -184,6 +187,17 @@ size_t qmoe_moe_workspace_bytes(int tokens, int top_k, int n_experts, int d_mode
  * there is no host round trip. */
 int qmoe_moe_forward(const qmoe_moe_args* args, void* workspace, size_t workspace_bytes,
                      void* stream);
+
+/* RMSNorm of the residual stream followed by the router's logits, the step in front of the MoE
+ * block, in one launch:  normalized = (x * inv_rms) * gamma  with  inv_rms = 1 / sqrt(mean(x^2) + eps)
+ * (RMSNormInference.forward, mini_llm/ops/rmsnorm_inference.py:109-118, :517-520) and
+ * logits = normalized @ router_w^T + router_b  (RouterInference.forward,
+ * mini_llm/ops/router_inference.py:40-46; router_w is [n_experts, d_model] as stored in
+ * ffn_gate_inp, router_b fp32 [n_experts] or NULL).  x [T, d_model], normalized [T, d_model] and
+ * logits [T, n_experts] are fp32; d_model % 4 == 0. */
+int qmoe_norm_router(const float* x, int tokens, int d_model, const float* gamma, float eps,
+                     const float* router_w, const float* router_b, int n_experts, float* normalized,
+                     float* logits, void* stream);
 
 #ifdef __cplusplus
 }

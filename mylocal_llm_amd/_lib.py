@@ -40,7 +40,7 @@ class MoeArgs(ctypes.Structure):
                 ("shared_gate_w", _P), ("shared_up_w", _P), ("shared_down_w", _P),
                 ("shared_gate_fmt", _I), ("shared_up_fmt", _I), ("shared_down_fmt", _I),
                 ("d_ff_shared", _I), ("shared_gate", _P),
-                ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P)]
+                ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P)]
 
 
 _SIGNATURES = {
@@ -56,6 +56,7 @@ _SIGNATURES = {
     "qmoe_grouped_decode": ([_P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _P, _P], _I),
     "qmoe_moe_workspace_bytes": ([_I, _I, _I, _I, _I, _I], _SZ),
     "qmoe_moe_forward": ([ctypes.POINTER(MoeArgs), _P, _SZ, _P], _I),
+    "qmoe_norm_router": ([_P, _I, _I, _P, _F, _P, _P, _I, _P, _P, _P], _I),
 }
 EXPORTS = tuple(_SIGNATURES)
 
@@ -82,7 +83,7 @@ def load():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes
                 fn.restype = restype
-            if lib.qmoe_abi_version() != 1:
+            if lib.qmoe_abi_version() != 2:
                 raise RuntimeError(f"{path}: unexpected ABI version {lib.qmoe_abi_version()}")
             _LIB = lib
         return _LIB

@@ -298,6 +298,7 @@ struct DecodeDownArgs {
     const float* sorted_w;      // [T, k]
     const float* sig;           // [T]
     void* out;                  // [T, D]
+    const float* residual;      // [T, D] added to the block's output, or null
     int odt, k, d, f, fsh, rows_per_wave;
 };
 
@@ -375,7 +376,10 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
                     const float y63 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ys), 63));
                     acc = add_product(acc, y63, sg);
                 }
-                if (lane == 0) store_out(a.out, a.odt, (size_t)t * a.d + row0 + r, acc);
+                if (lane == 0) {
+                    if (a.residual) acc = a.residual[(size_t)t * a.d + row0 + r] + acc;
+                    store_out(a.out, a.odt, (size_t)t * a.d + row0 + r, acc);
+                }
                 ++r;
                 if (r >= nrows) done = true;
             }
@@ -493,6 +497,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     d.sorted_w = w.sorted_w;
     d.sig = w.sig;
     d.out = a.out;
+    d.residual = a.residual;
     d.odt = a.out_dtype;
     d.k = a.top_k;
     d.d = b.d_model;

@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                                                           const float* __restrict__ shared_out,
                                                           const float* __restrict__ shared_gate,
                                                           const void* __restrict__ x, void* __restrict__ out,
-                                                          int odt) {
+                                                          int odt, const float* __restrict__ residual) {
     __shared__ int order[32];
     __shared__ float partial[4];
     __shared__ float sigmoid;
@@ -261,6 +261,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                 acc.x = add_product(acc.x, v.x, sg); acc.y = add_product(acc.y, v.y, sg);
                 acc.z = add_product(acc.z, v.z, sg); acc.w = add_product(acc.w, v.w, sg);
             }
+            if (residual) {
+                const float4 r = *(const float4*)(residual + (size_t)t * d + i);
+                acc.x = __fadd_rn(r.x, acc.x); acc.y = __fadd_rn(r.y, acc.y);
+                acc.z = __fadd_rn(r.z, acc.z); acc.w = __fadd_rn(r.w, acc.w);
+            }
             store_out(out, odt, (size_t)t * d + i, acc.x);
             store_out(out, odt, (size_t)t * d + i + 1, acc.y);
             store_out(out, odt, (size_t)t * d + i + 2, acc.z);
@@ -275,6 +280,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
             if (p >= 0) acc = __fadd_rn(acc, terms[(size_t)p * d + i]);
         }
         if (shared_out) acc = add_product(acc, shared_out[(size_t)t * d + i], sg);
+        if (residual) acc = __fadd_rn(residual[(size_t)t * d + i], acc);
         store_out(out, odt, (size_t)t * d + i, acc);
     }
 }
@@ -583,7 +589,7 @@ static int launch_combine(const qmoe_moe_args& a, char* ws, const MoeWorkspace& 
 #define QMOE_COMBINE(XDT)                                                                                            \
     hipLaunchKernelGGL((moe_combine_kernel<XDT>), cgrid, cblock, 0, s, (const float*)(ws + L.terms),                 \
                        (const int*)(ws + L.pos_of), a.top_k, b.d_model, shared_out, a.shared_gate, a.hidden, a.out,  \
-                       a.out_dtype)
+                       a.out_dtype, a.residual)
     if (a.hidden_dtype == QMOE_DT_F32) QMOE_COMBINE(QMOE_DT_F32);
     else if (a.hidden_dtype == QMOE_DT_F16) QMOE_COMBINE(QMOE_DT_F16);
     else QMOE_COMBINE(QMOE_DT_BF16);

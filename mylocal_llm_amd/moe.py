@@ -131,16 +131,45 @@ def _max_tokens_per_call(n_experts):
     return words * 32
 
 
+def norm_router(x, gamma, eps, router_weight, router_bias=None):
+    """RMSNorm of fp32 ``x`` [T, D] followed by the router's logits, in one launch.
+
+    Returns ``(normalized [T, D], logits [T, E])``: ``normalized = (x * inv_rms) * gamma`` as
+    RMSNormInference.forward computes it (mini_llm/ops/rmsnorm_inference.py:109-118) and
+    ``logits = normalized @ router_weight.T (+ bias)`` (mini_llm/ops/router_inference.py:40-46);
+    ``router_weight`` is fp32 [E, D], the orientation of the checkpoint's ``ffn_gate_inp``.
+    """
+    for name, tensor in (("x", x), ("gamma", gamma), ("router_weight", router_weight)):
+        if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda or tensor.dtype != torch.float32 or not tensor.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous CUDA float32 tensor")
+    if x.ndim != 2 or gamma.shape != (x.shape[1],) or router_weight.ndim != 2 or router_weight.shape[1] != x.shape[1]:
+        raise ValueError("x [T, D], gamma [D] and router_weight [E, D] do not fit together")
+    t, d = x.shape
+    e = router_weight.shape[0]
+    if router_bias is not None and (router_bias.dtype != torch.float32 or tuple(router_bias.shape) != (e,) or not router_bias.is_cuda):
+        raise ValueError("router_bias must be CUDA float32 [E]")
+    normalized = torch.empty_like(x)
+    logits = torch.empty((t, e), dtype=torch.float32, device=x.device)
+    if t:
+        with torch.cuda.device(x.device):
+            rc = _lib.load().qmoe_norm_router(_ptr(x), t, d, _ptr(gamma), float(eps), _ptr(router_weight),
+                                              _ptr(router_bias) if router_bias is not None else _NULL, e,
+                                              _ptr(normalized), _ptr(logits), _stream())
+        _lib.check(rc, "RMSNorm + router logits")
+    return normalized, logits
+
+
 def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared=None,
              shared_gate=None, floor=2.0 ** -14, renormalize=True, out_dtype=None,
-             return_routing=False):
+             return_routing=False, residual=None):
     """One MoE step over hidden [T, D]: routed experts (+ shared expert) -> [T, D].
 
     Routing comes from fp32 ``logits`` [T, E] (softmax/top-k on the device) or from
     precomputed ``weights`` fp32 / ``ids`` int64 [T, k].  ``shared`` is an optional
     (gate, up, down) triple of DevicePackedGGUFWeight; ``shared_gate`` an optional fp32 [D]
     admission vector (sigmoid gate).  Accumulation is fp32; the output is rounded once to
-    ``out_dtype`` (default: hidden's dtype).
+    ``out_dtype`` (default: hidden's dtype).  ``residual`` (optional fp32 [T, D]) is added to the
+    block's output in the same kernels: ``residual + (routed + shared * sigmoid)``.
     """
     if not isinstance(hidden, torch.Tensor) or not hidden.is_cuda or hidden.dtype not in _TORCH_DTYPE_ID:
         raise TypeError("MoE hidden must be a CUDA FP16/BF16/FP32 tensor")
@@ -159,6 +188,9 @@ def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared
                 or tuple(weights.shape) != (t, top_k) or tuple(ids.shape) != (t, top_k)
                 or not weights.is_contiguous() or not ids.is_contiguous()):
             raise ValueError("routing weights / ids must be contiguous FP32 / int64 [tokens, k]")
+    if residual is not None and (not isinstance(residual, torch.Tensor) or residual.dtype != torch.float32 or not residual.is_cuda
+                                 or tuple(residual.shape) != (t, bank.d_model) or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous CUDA FP32 [tokens, d_model]")
     out_w = torch.empty((t, top_k), dtype=torch.float32, device=hidden.device) if return_routing else None
     out_i = torch.empty((t, top_k), dtype=torch.int64, device=hidden.device) if return_routing else None
     if t == 0:
@@ -191,6 +223,8 @@ def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared
                 if shared_gate is not None:
                     args.shared_gate = shared_gate.data_ptr()
             args.out, args.out_dtype = out[lo:hi].data_ptr(), _TORCH_DTYPE_ID[out_dtype]
+            if residual is not None:
+                args.residual = residual[lo:hi].data_ptr()
             if return_routing:
                 args.out_weights, args.out_ids = out_w[lo:hi].data_ptr(), out_i[lo:hi].data_ptr()
             rc = lib.qmoe_moe_forward(ctypes.byref(args), _ptr(workspace), nbytes, _stream())
@@ -311,7 +345,8 @@ class Qwen3NextMoEInference:
         self.top_k = int(top_k)
         self.router = RouterInference(bank.d_model, bank.n_experts, self.top_k,
                                       renormalize_selected=True, normalization_floor=normalization_floor)
-        self.router.W_router = router_weight.to(torch.float32).t().contiguous()
+        self._router_weight = router_weight.to(torch.float32).contiguous()  # [E, D], as stored
+        self.router.W_router = self._router_weight.t().contiguous()
         self.router.b_router = torch.zeros(bank.n_experts, dtype=torch.float32, device=router_weight.device)
         self.shared_is_dense = all(isinstance(w, torch.Tensor) for w in shared)
         if not self.shared_is_dense and not all(isinstance(w, DevicePackedGGUFWeight) for w in shared):
@@ -347,6 +382,26 @@ class Qwen3NextMoEInference:
         result = cls(bank, spec.top_k, dense('ffn_gate_inp.weight'), shared, dense('ffn_gate_inp_shexp.weight'))
         result.index, result.layer_id, result.spec = index, layer_id, spec
         return result
+
+    def forward_after_norm(self, residual, gamma, eps):
+        """``residual + forward(rmsnorm(residual))``: the second half of a decoder layer
+        (mini_llm/external/qwen3next_decoder.py:120) with the norm and the router's logits in one
+        launch in front of the block and the residual add inside its last kernels."""
+        if not isinstance(residual, torch.Tensor) or residual.dtype != torch.float32:
+            raise TypeError('Qwen3-Next MoE requires backend float32 hidden')
+        if residual.ndim != 3 or residual.shape[0] < 1 or residual.shape[-1] != self.bank.d_model:
+            raise ValueError('hidden must have shape [positive batch,time,d_model]')
+        if not residual.shape[1]:
+            return residual.clone()
+        if self.shared_is_dense:
+            normalized, _ = norm_router(residual.reshape(-1, residual.shape[-1]).contiguous(), gamma, eps, self._router_weight)
+            return residual + self.forward(normalized.reshape(residual.shape))
+        b, t, d = residual.shape
+        flat = residual.reshape(b * t, d).contiguous()
+        normalized, logits = norm_router(flat, gamma, eps, self._router_weight)
+        out = moe_step(normalized, self.bank, self.top_k, logits=logits, shared=self.shared, shared_gate=self.shared_gate,
+                       floor=self.router.normalization_floor, residual=flat)
+        return out.reshape(b, t, d)
 
     def forward(self, hidden):
         if not isinstance(hidden, torch.Tensor) or hidden.dtype != torch.float32:

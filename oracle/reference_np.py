@@ -351,6 +351,22 @@ def moe_forward(hidden, logits, k, n_experts, expert_fn, shared, shared_gate, *,
     return routed + sh * sig[..., None], w, ids
 
 
+def rmsnorm(x, gamma, eps):
+    """``(x * inv_rms) * gamma`` with ``inv_rms = 1 / sqrt(mean(x*x) + eps)`` in fp32
+    (mini_llm/ops/rmsnorm_inference.py:517-520; the fused kernel :109-118 has the same graph)."""
+    x = np.asarray(x, np.float32)
+    mean_sq = np.mean(x * x, axis=-1, keepdims=True, dtype=np.float32)
+    inv_rms = np.float32(1.0) / np.sqrt(mean_sq + np.float32(eps))
+    return (x * inv_rms) * np.asarray(gamma, np.float32)
+
+
+def router_logits(x, router_weight, bias=None):
+    """``x @ W_router + b`` with ``W_router = router_weight.T`` (router_weight is [E, D] as stored in
+    ffn_gate_inp; mini_llm/ops/router_inference.py:40-46, qwen3next_moe.py:111-113), fp32."""
+    out = np.asarray(x, np.float32) @ np.asarray(router_weight, np.float32).T
+    return out if bias is None else out + np.asarray(bias, np.float32)
+
+
 PINNING = {
     "dequantize/Q8_0": "closed form d*int8; large-output vector of tests/test_0106p (q=(row%15-7), d=.125)",
     "dequantize/Q4_0": "hand-packed vector of tests/test_0106a:18-25",
@@ -362,6 +378,8 @@ PINNING = {
     "all formats": "cross-check against oracle/_ref (the reference's own C++ packed dot, identity rows) where it builds",
     "linear": "textbook fp32 GEMV; checked against an fp64 matmul of the dequantised matrix",
     "swiglu / expert_ffn": "closed form; fp64 matched-storage formula of diagnostics/quantized_numerics.py:42-59",
+    "rmsnorm": "closed forms (constant rows -> gamma*c/sqrt(c*c+eps); eps=0 scale invariance) and an fp64 evaluation",
+    "router_logits": "textbook fp32 GEMV against an fp64 matmul",
     "router_topk": "tie / inf / NaN fixtures of tests/test_0106v:44-62; sum(w)=1 when mass>=floor; ids unique",
     "experts_forward / grouped_decode": "ordered-sum cancellation fixtures (1e8,1,-1e8,3 -> 3) of tests/test_0106t:321-330; brute-force per-token loop",
     "moe_forward": "independent fp64 per-token loop after tests/test_0106o_qwen3next_decoder:103-127; zero gate -> x0.5",

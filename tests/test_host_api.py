@@ -75,7 +75,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.EXPORTS)
     for name in names:
         assert getattr(lib, name) is not None
-    assert lib.qmoe_abi_version() == 1
+    assert lib.qmoe_abi_version() == 2
 
 
 def test_format_info_matches_table():

@@ -241,3 +241,28 @@ def test_moe_forward_against_independent_fp64_loop():
                                lambda e, rows: R.expert_ffn(rows, *experts[e]), shared, np.zeros_like(gate_vec))
     np.testing.assert_allclose(out0, expect0, rtol=3e-4, atol=3e-5 * scale)
     np.testing.assert_array_equal(R.shared_gate_sigmoid(hidden, np.zeros_like(gate_vec)), np.full(hidden.shape[0], .5, np.float32))
+
+
+def test_rmsnorm_closed_forms_and_fp64():
+    d = 96
+    gamma = np.linspace(0.5, 1.5, d).astype(np.float32)
+    for c, eps in ((3.0, 1e-6), (-0.25, 1e-5), (1e-3, 1e-6)):
+        row = np.full((2, d), c, np.float32)
+        want = gamma.astype(np.float64) * c / np.sqrt(c * c + eps)
+        np.testing.assert_allclose(R.rmsnorm(row, gamma, eps)[1], want, rtol=3e-7)
+    x = np.random.default_rng(3).standard_normal((5, d)).astype(np.float32)
+    np.testing.assert_allclose(R.rmsnorm(4.0 * x, gamma, 0.0), R.rmsnorm(x, gamma, 0.0), rtol=1e-6)   # scale invariance at eps = 0
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt(np.mean(x64 * x64, axis=-1, keepdims=True) + 1e-6) * gamma
+    got = R.rmsnorm(x, gamma, 1e-6)
+    assert got.dtype == np.float32
+    np.testing.assert_allclose(got, want, rtol=1e-6)
+    # a dropped eps, a mean taken as a sum or gamma left out each fail one of the above
+    assert not np.allclose(R.rmsnorm(np.full((1, d), 1e-3, np.float32), gamma, 1e-6), gamma)
+
+
+def test_router_logits_against_fp64():
+    rng = np.random.default_rng(4)
+    x, w, b = rng.standard_normal((3, 128)).astype(np.float32), rng.standard_normal((16, 128)).astype(np.float32), rng.standard_normal(16).astype(np.float32)
+    np.testing.assert_allclose(R.router_logits(x, w, b), x.astype(np.float64) @ w.astype(np.float64).T + b, rtol=1e-5, atol=1e-5)
+    assert R.router_logits(x, w).shape == (3, 16)
