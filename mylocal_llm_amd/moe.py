@@ -233,15 +233,24 @@ def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared
 
 
 class ExpertsInference:
-    """Sparse expert dispatch + ordered weighted combine over an HBM-resident bank."""
+    """Sparse expert dispatch + ordered weighted combine.
+
+    ``expert_executor`` is either a resident ``DevicePackedExpertBank`` (the layer's experts) or an
+    executor with the hooks of the reference's (mini_llm/ops/experts_inference.py:188-197:
+    ``try_forward_device_plan`` for one token; this package's executor also offers
+    ``try_forward_batch`` for more), e.g. ``expert_executor.ResidentExpertExecutor``.
+    """
 
     def __init__(self, d_model, d_ff, n_experts, dtype="float32", *, expert_executor=None, layer_id=0):
         self.d_model, self.d_ff, self.n_experts = d_model, d_ff, n_experts
         self.layer_id = int(layer_id)
-        # The "executor" of this build is the resident bank itself.
-        self.bank = expert_executor
-        if self.bank is not None and (self.bank.d_model, self.bank.d_ff, self.bank.n_experts) != (d_model, d_ff, n_experts):
-            raise ValueError("Executor dimensions do not match MoE tensors")
+        self.bank = self.expert_executor = None
+        if isinstance(expert_executor, DevicePackedExpertBank):
+            self.set_bank(expert_executor)
+        elif expert_executor is not None:
+            if (expert_executor.d_model, expert_executor.d_ff) != (d_model, d_ff):
+                raise ValueError("Executor dimensions do not match MoE tensors")
+            self.expert_executor = expert_executor
 
     def set_bank(self, bank):
         if (bank.d_model, bank.d_ff, bank.n_experts) != (self.d_model, self.d_ff, self.n_experts):
@@ -250,12 +259,30 @@ class ExpertsInference:
 
     def forward(self, x, weights, expert_indices, *, on_cpu_submitted=None):
         """y[tok] = sum over its experts, ascending id, of w * expert(x[tok]); x is [B, T, D]."""
-        if self.bank is None:
-            raise RuntimeError("ExpertsInference has no resident expert bank")
         batch_size, seq_len, d_model = x.shape
         k = weights.shape[-1]
         n = batch_size * seq_len
-        y = moe_step(x.reshape(n, d_model).contiguous(), self.bank, k,
+        flat = x.reshape(n, d_model).contiguous()
+        if self.expert_executor is not None:
+            ex = self.expert_executor
+            y = None
+            if n == 1 and getattr(ex, "try_forward_device_plan", None) is not None:
+                args = (self.layer_id, flat, weights.reshape(-1), expert_indices.reshape(-1), self.n_experts)
+                y = (ex.try_forward_device_plan(*args, on_cpu_submitted=on_cpu_submitted) if on_cpu_submitted is not None
+                     else ex.try_forward_device_plan(*args))
+                if y is not None:
+                    return y.reshape(batch_size, seq_len, d_model)
+            batch = getattr(ex, "try_forward_batch", None)
+            if batch is None:
+                raise RuntimeError("the expert executor offers neither try_forward_device_plan for this call nor try_forward_batch")
+            with ex.dispatch_scope(self.layer_id, ()):
+                y = batch(self.layer_id, flat, weights.reshape(n, k), expert_indices.reshape(n, k))
+            if on_cpu_submitted is not None:
+                on_cpu_submitted()
+            return y.reshape(batch_size, seq_len, d_model)
+        if self.bank is None:
+            raise RuntimeError("ExpertsInference has no resident expert bank")
+        y = moe_step(flat, self.bank, k,
                      weights=weights.reshape(n, k).to(torch.float32).contiguous(),
                      ids=expert_indices.reshape(n, k).to(torch.int64).contiguous())
         if on_cpu_submitted is not None:
@@ -359,13 +386,20 @@ class Qwen3NextMoEInference:
     def from_index(cls, index, layer_id, *, expert_executor=None, device=None):
         """Build the block of ``layer_id`` from a ``Qwen3NextGGUFIndex``
         (mini_llm/external/qwen3next_moe.py:100-127).  ``expert_executor`` may be a resident
-        ``DevicePackedExpertBank`` the caller already holds for this layer; otherwise the
-        layer's routed tensors are uploaded."""
+        ``DevicePackedExpertBank`` the caller already holds for this layer or an executor that
+        holds it (``ResidentExpertExecutor``); otherwise the layer's routed tensors are uploaded."""
         spec = Qwen3NextMoESpec.from_index(index, layer_id)
         if not torch.cuda.is_available():
             raise RuntimeError('Packed GPU weights require a HIP device')
         dev = torch.device('cuda', torch.cuda.current_device()) if device is None else torch.device(device)
-        bank = expert_executor if expert_executor is not None else index.expert_bank(layer_id, dev)
+        if expert_executor is None:
+            bank = index.expert_bank(layer_id, dev)
+        elif isinstance(expert_executor, DevicePackedExpertBank):
+            bank = expert_executor
+        else:  # an executor holding this layer's bank (expert_executor.ResidentExpertExecutor)
+            if getattr(expert_executor, 'compute_dtype', 'float32') != 'float32':
+                raise ValueError('Qwen3-Next adapter requires float32 expert compute')
+            bank = expert_executor.bank(layer_id)
         if (bank.d_model, bank.d_ff) != (spec.d_model, spec.d_ff) or bank.n_experts != spec.n_experts:
             raise ValueError('Executor dimensions do not match MoE tensors')
         stem = f'blk.{layer_id}.'
