@@ -260,10 +260,8 @@ def moe_prefill_extra(torch, lib, device, fmt, tokens, steps, warmup):
     calls = []
     for i in range(n_banks):
         a = _lib.MoeArgs()
-        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), hdt, tokens, k
+        a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), 2, tokens, k
         a.logits, a.floor_value, a.renormalize = logits[i].data_ptr(), 2.0 ** -14, 1
-        if layer_half:
-            a.residual = residual.data_ptr()
         banks[i].fill(a.bank)
         g, u, dn = shareds[i]
         a.shared_gate_w, a.shared_up_w, a.shared_down_w = g.data.data_ptr(), u.data.data_ptr(), dn.data.data_ptr()
