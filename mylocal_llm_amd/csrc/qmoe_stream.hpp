@@ -453,8 +453,21 @@ __device__ __forceinline__ void stream_problem(const StreamProblem& p, float* pa
     // New activations are staged once per workgroup in LDS (as fp32) while this wave's first
     // rows are already in flight; every wave of the workgroup passes here for every problem.
     if (staged != p.xgroup) {
+        // all loads first, then all LDS stores: the loads travel together (a store between two
+        // loads would order them, LDS and global pointers are not told apart here), and they
+        // travel while the workgroup's other waves are still finishing what reads the old contents
+        float4 v[STREAM_MAX_K / (4 * STREAM_THREADS)];
+#pragma unroll
+        for (int j = 0; j < STREAM_MAX_K / (4 * STREAM_THREADS); ++j) {
+            const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+            if (i < p.k) v[j] = load_x4(p.x, p.xdt, i);
+        }
         __syncthreads();
-        for (int i = 4 * threadIdx.x; i < p.k; i += 4 * STREAM_THREADS) *(float4*)(xs + StagedX::at(i)) = load_x4(p.x, p.xdt, i);
+#pragma unroll
+        for (int j = 0; j < STREAM_MAX_K / (4 * STREAM_THREADS); ++j) {
+            const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+            if (i < p.k) *(float4*)(xs + StagedX::at(i)) = v[j];
+        }
         __syncthreads();
         staged = p.xgroup;
     }
@@ -629,10 +642,16 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
                     } else {
                         const uint8_t* px = uniform((const uint8_t*)p.x);
                         const int pxdt = uniform(p.xdt);
+                        float4 v[16];  // all loads first, then all LDS stores
 #pragma unroll
                         for (int i = 0; i < 16; ++i) {
                             const int idx = 4 * lane + 256 * i;
-                            if (idx < pk) *(float4*)(xw + StagedX::at(idx)) = load_x4(px, pxdt, idx);
+                            if (idx < pk) v[i] = load_x4(px, pxdt, idx);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            const int idx = 4 * lane + 256 * i;
+                            if (idx < pk) *(float4*)(xw + StagedX::at(idx)) = v[i];
                         }
                     }
                     U::load_x(StagedX{xl}, active ? u : 0, xr, aux);
