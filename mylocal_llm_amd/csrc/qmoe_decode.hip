@@ -194,9 +194,20 @@ __device__ __forceinline__ void shared_pairs_phase(const DecodeRouteArgs& a, flo
     for (int t0 = 0; t0 < a.tokens; t0 += fit) {
         const int groups = a.tokens - t0 < fit ? a.tokens - t0 : fit;
         __syncthreads();
-        for (int g = 0; g < groups; ++g)
-            for (int i = 4 * threadIdx.x; i < a.d; i += 4 * STREAM_THREADS)
-                *(float4*)(xs + g * stripe + StagedX::at(i)) = load_x4(a.hidden, a.xdt, (t0 + g) * a.d + i);
+        // a token's loads are issued together, then stored (a store between two loads orders them)
+        for (int g = 0; g < groups; ++g) {
+            float4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+                if (i < a.d) v[j] = load_x4(a.hidden, a.xdt, (t0 + g) * a.d + i);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+                if (i < a.d) *(float4*)(xs + g * stripe + StagedX::at(i)) = v[j];
+            }
+        }
         __syncthreads();
         stream_rows_many_x<FMT, true, Prefetch<FMT, true>::DEPTH>(a.shared_gate_w, a.shared_up_w, a.fsh, a.d, xs, stripe, groups,
                                                                  a.hs + (size_t)t0 * a.fsh, a.fsh,
@@ -341,8 +352,21 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
     const int nr = k * a.f, total = nr + (a.shared_down ? a.fsh : 0);
     const float* hr = a.h + (size_t)t * nr;
     const float* hsh = a.hs + (size_t)t * a.fsh;
-    for (int i = 4 * threadIdx.x; i < total; i += 4 * 256)
-        *(float4*)(xs + StagedX::at(i)) = i < nr ? *(const float4*)(hr + i) : *(const float4*)(hsh + (i - nr));
+    {
+        // all loads first, then the LDS stores (a store between two loads orders them)
+        constexpr int NV = 8192 / (4 * 256);
+        float4 v[NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = 4 * threadIdx.x + 4 * 256 * j;
+            if (i < total) v[j] = i < nr ? ldg<float4>(hr + i) : ldg<float4>(hsh + (i - nr));
+        }
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = 4 * threadIdx.x + 4 * 256 * j;
+            if (i < total) *(float4*)(xs + StagedX::at(i)) = v[j];
+        }
+    }
     __syncthreads();
     const int ux = shared ? (nr >> 6) + 2 * part : slot * (a.f >> 6) + 2 * part;
     float x0[64], x1[64], aux0[U::AUX], aux1[U::AUX];
