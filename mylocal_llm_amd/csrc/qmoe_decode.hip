@@ -226,8 +226,47 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     if (a.shared_apart) shared_pairs_phase<FMT>(a, xs);
     const int n = *count;
-    // descriptors are fetched a stage at a time by the whole workgroup, not one dependent
-    // load per problem
+    const int units = a.d >> 6;
+    if (units <= 64) {
+        // Rows that fit a wave: tokens are taken in groups whose activations fit the LDS stripes
+        // (eight tokens of 2048 columns) and whose descriptors fit the staging array; inside a
+        // group the waves sweep the item stream together (item w, w + W, ...), as in the fused
+        // kernel, instead of each wave walking a stretch of its own.
+        const int per_token = a.k + ((a.shared_gate_w && !a.shared_apart) ? 1 : 0);
+        const int stripe = a.d + 4 * units;
+        int group = STREAM_XS_FLOATS / stripe;
+        if (group > LIST_STAGE / per_token) group = LIST_STAGE / per_token;
+        for (int t0 = 0; t0 < a.tokens; t0 += group) {
+            const int nt = a.tokens - t0 < group ? a.tokens - t0 : group;
+            const int base = t0 * per_token;
+            int m = nt * per_token;
+            if (base + m > n) m = n - base;
+            if (m <= 0) break;
+            __syncthreads();
+            const uint4* src = (const uint4*)(list + base);
+            uint4* dst = (uint4*)staged;
+            for (int i = threadIdx.x; i < m * 4; i += STREAM_THREADS) dst[i] = src[i];
+            for (int g = 0; g < nt; ++g) {
+                float4 v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+                    if (i < a.d) v[j] = load_x4(a.hidden, a.xdt, (t0 + g) * a.d + i);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+                    if (i < a.d) *(float4*)(xs + g * stripe + StagedX::at(i)) = v[j];
+                }
+            }
+            __syncthreads();
+            if ((int)threadIdx.x < m) staged[threadIdx.x].xgroup -= t0;   // stripe of the token inside this group
+            __syncthreads();
+            stream_run<FMT, PAIR, false>(staged, m, staged[0].first_item, staged[m - 1].flat_end, false, partial, xs, xs, stripe);
+        }
+        return;
+    }
+    // wider rows: descriptors are fetched a stage at a time by the whole workgroup, four waves a row
     for (int base = 0; base < n; base += LIST_STAGE) {
         const int m = n - base < LIST_STAGE ? n - base : LIST_STAGE;
         __syncthreads();
@@ -235,9 +274,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
         uint4* dst = (uint4*)staged;
         for (int i = threadIdx.x; i < m * 4; i += STREAM_THREADS) dst[i] = src[i];
         __syncthreads();
-        // the stage's share of the flat item stream (empty when the rows are wider than a wave)
-        const int wide = (staged[0].k >> 6) > 64;
-        stream_run<FMT, PAIR>(staged, m, wide ? 0 : staged[0].first_item, wide ? 0 : staged[m - 1].flat_end, true, partial, xs);
+        stream_run<FMT, PAIR>(staged, m, 0, 0, true, partial, xs);
     }
 }
 

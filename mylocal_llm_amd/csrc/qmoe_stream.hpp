@@ -562,10 +562,11 @@ __device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
 // so the start of a new matrix does not drain the memory pipeline.
 // Activations are fetched coalesced into the wave's private LDS stripe `xw` and read back as
 // the lane's 64-value slice; with `xpre` the caller has already put the activations of
-// xgroup g into stripe g of that array (same padded layout) and nothing is fetched here.  Items [begin, end) are walked; `probs` covers them in order.
+// xgroup g into stripe g of that array (same padded layout, stripes `xstride` floats apart) and
+// nothing is fetched here.  Items [begin, end) are walked; `probs` covers them in order.
 template <int FMT, bool PAIR, int PD>
 __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, bool contiguous, float* xw,
-                                            const float* xpre) {
+                                            const float* xpre, int xstride = STREAM_XS_FLOATS / STREAM_WAVES) {
     using U = Unit64<FMT>;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = gridDim.x * STREAM_WAVES;
@@ -638,7 +639,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
                 if (xgroup != pg) {
                     const float* xl = xw;
                     if (xpre) {
-                        xl = xpre + pg * (STREAM_XS_FLOATS / STREAM_WAVES);
+                        xl = xpre + pg * xstride;
                     } else {
                         const uint8_t* px = uniform((const uint8_t*)p.x);
                         const int pxdt = uniform(p.xdt);
@@ -738,11 +739,11 @@ template <int FMT, bool PAIR> struct Prefetch {
 // wave, then, one after the other, the problems with wider rows (four waves per row).
 template <int FMT, bool PAIR, bool WIDE = true>
 __device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, bool contiguous, float* partial, float* xs,
-                                           const float* xpre = nullptr) {
+                                           const float* xpre = nullptr, int xstride = STREAM_XS_FLOATS / STREAM_WAVES) {
     constexpr int PD = Prefetch<FMT, PAIR>::DEPTH;
     const int wave = threadIdx.x >> 6;
     if (flat_end > flat_begin)
-        stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES), xpre);
+        stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES), xpre, xstride);
     if (!WIDE) return;
     float xr[64], aux[8];
     int xgroup = -1, staged = -1;
