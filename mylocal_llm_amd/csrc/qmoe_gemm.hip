@@ -13,8 +13,11 @@
 //     eight v_mfma_f32_16x16x32_bf16 steps, with no LDS round trip for weights;
 //   * hi*hi + lo*hi + hi*lo accumulate in fp32 (lo*lo is below 2^-32 of the product).
 // Rows of the next pass (weights and activations) are requested before the current pass is
-// multiplied.
+// multiplied.  Q8_0 takes its own loop (q8_tile_loop below): whole weight tiles go through LDS
+// and the integer codes themselves are the B operand.
 #include "qmoe_gemm.hpp"
+
+#include <type_traits>
 
 #include "qmoe_mfma.hpp"
 #include "qmoe_stream.hpp"
@@ -22,6 +25,12 @@
 namespace qmoe {
 
 static constexpr int GEMM_THREADS = 256;
+#ifndef QMOE_BF16_WGS
+#define QMOE_BF16_WGS 3
+#endif
+#ifndef QMOE_PLAIN_NM
+#define QMOE_PLAIN_NM 1
+#endif
 static constexpr int GEMM_A_STRIDE = 528;                       // bytes of one staged token row
 static constexpr int GEMM_TERM_BYTES = GEMM_CHUNK * GEMM_A_STRIDE;  // one bf16 term of the chunk
 
@@ -30,22 +39,21 @@ template <int AKIND> struct AStage {
 };
 
 // Eight consecutive columns of one activation row, as they lie in memory; a position outside
-// the chunk or the row reads (valid) element 0 instead and is replaced by zeros.
+// the chunk or the row reads (valid) element 0 instead.  The caller zeroes such a position when
+// it stores, so that no load has to be waited for where it is issued.
 template <int AKIND>
-__device__ __forceinline__ void stage_load(uint4& r0, uint4& r1, const GemmArgs& a, int64_t row, int col, bool valid) {
+__device__ __forceinline__ void stage_fetch(uint4& r0, uint4& r1, const GemmArgs& a, int64_t row, int col, bool valid) {
     const int64_t at = valid ? row * a.a_stride + col : 0;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
     if (AKIND == GEMM_A_F32) {
-        r0 = *(const uint4*)((const float*)a.a0 + at);
-        r1 = *(const uint4*)((const float*)a.a0 + at + 4);
+        r0 = ldg<uint4>((const float*)a.a0 + at);
+        r1 = ldg<uint4>((const float*)a.a0 + at + 4);
     } else if (AKIND == GEMM_A_PAIR) {
-        r0 = *(const uint4*)((const uint16_t*)a.a0 + at);
-        r1 = *(const uint4*)((const uint16_t*)a.a1 + at);
+        r0 = ldg<uint4>((const uint16_t*)a.a0 + at);
+        r1 = ldg<uint4>((const uint16_t*)a.a1 + at);
     } else {
-        r0 = *(const uint4*)((const uint16_t*)a.a0 + at);
-        r1 = zero;
+        r0 = ldg<uint4>((const uint16_t*)a.a0 + at);
+        r1 = make_uint4(0, 0, 0, 0);
     }
-    if (!valid) { r0 = zero; r1 = zero; }
 }
 
 // ... and their bf16 terms into the staged tile (hi at `dst`, lo TERM bytes further).
@@ -74,16 +82,242 @@ __device__ __forceinline__ void stage_store(const uint4 r0, const uint4 r1, uint
     }
 }
 
+// The two bf16 terms of eight staged columns, as 16 bytes each.
+template <int AKIND>
+__device__ __forceinline__ void stage_terms(const uint4 r0, const uint4 r1, uint4& hi, uint4& lo) {
+    if (AKIND == GEMM_A_BF16) {
+        hi = r0;
+        lo = make_uint4(0, 0, 0, 0);
+    } else if (AKIND == GEMM_A_PAIR) {
+        hi = r0;
+        lo = r1;
+    } else {
+        float v[8];
+        if (AKIND == GEMM_A_F32) {
+            v[0] = __uint_as_float(r0.x); v[1] = __uint_as_float(r0.y); v[2] = __uint_as_float(r0.z); v[3] = __uint_as_float(r0.w);
+            v[4] = __uint_as_float(r1.x); v[5] = __uint_as_float(r1.y); v[6] = __uint_as_float(r1.z); v[7] = __uint_as_float(r1.w);
+        } else {
+            v[0] = half_bits_to_float(r0.x & 0xFFFFu); v[1] = half_bits_to_float(r0.x >> 16);
+            v[2] = half_bits_to_float(r0.y & 0xFFFFu); v[3] = half_bits_to_float(r0.y >> 16);
+            v[4] = half_bits_to_float(r0.z & 0xFFFFu); v[5] = half_bits_to_float(r0.z >> 16);
+            v[6] = half_bits_to_float(r0.w & 0xFFFFu); v[7] = half_bits_to_float(r0.w >> 16);
+        }
+        OperandBits h, l;
+        split_terms(v, h, l);
+        hi = make_uint4(h.u[0], h.u[1], h.u[2], h.u[3]);
+        lo = make_uint4(l.u[0], l.u[1], l.u[2], l.u[3]);
+    }
+}
+
+// ---- Q8_0: weight tiles through LDS, integer codes as the MFMA operand ---------------------------
+// A Q8_0 weight is d * q with q an int8, and every int8 is a bf16 exactly.  So the B operand is
+// the codes themselves (one bf16 term, one conversion per code) and the block scale multiplies
+// the 32-column partial product afterwards: acc += d[row, block] * sum_k q[row, k] * x[token, k],
+// which is the same sum the dequantised weights give.  The workgroup copies the 272 bytes that
+// hold 256 columns of each of its rows from global memory to LDS with 16-byte loads that cover
+// whole cache lines once, and every wave takes its operands from there.
+// Within a block of 32 columns lane group g multiplies columns 4g..4g+3 and 16+4g..16+4g+3: two
+// dwords of codes per lane that the four groups of a row read from neighbouring LDS banks.
+// The staged activations are laid out to match (Q8Perm).
+static constexpr int Q8_SEG = 272;   // bytes of 256 columns of one row
+static constexpr int Q8_ROW = 272;   // bytes between staged rows in LDS
+template <int NM> struct Q8Tile {
+    static constexpr int ROWS = 64 * NM, CHUNKS = ROWS * 17, SLOTS = (CHUNKS + GEMM_THREADS - 1) / GEMM_THREADS;
+    static constexpr int BYTES = ROWS * Q8_ROW;
+};
+
+// four int8 codes -> four bf16 (exact)
+__device__ __forceinline__ void q8_codes_to_bf16(uint32_t q, uint32_t& lo2, uint32_t& hi2) {
+    const float f0 = (float)(int)(int8_t)(q & 0xFF), f1 = (float)(int)(int8_t)((q >> 8) & 0xFF);
+    const float f2 = (float)(int)(int8_t)((q >> 16) & 0xFF), f3 = (float)(int)(int8_t)(q >> 24);
+    lo2 = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+    hi2 = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+}
+
+// The workgroup walks `nblocks` row blocks from `rowblock` on for the same chunk: the weights of
+// the next pass are requested while the current one is multiplied, across row blocks as well, so
+// the wait for the first bytes is paid once per workgroup; emit(block) stores a finished block.
+template <int AKIND, bool PAIR, int NM, int MT, class Emit>
+__device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start, int count, int rowblock, int nblocks,
+                                             uint8_t* lds, floatx4 (&acc)[NM][MT], Emit emit) {
+    constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
+    constexpr int TERM = GEMM_TERM_BYTES;
+    using TL = Q8Tile<NM>;
+    uint8_t* wt = lds + NA * GEMM_TERM_BYTES;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 15, g = lane >> 4;
+    const int passes = (a.k + 255) >> 8;
+    const int rb = (a.k >> 5) * 34;
+    // this thread's 16-byte pieces of the weight tile: piece tid + 256*i lies 16 bytes a piece in LDS
+    // (272 = 17 * 16) and comes from byte woff[i] + piece[i] behind the matrix of its row
+    const uint8_t* const base0 = a.w + (int64_t)e * a.stride;
+    const uint8_t* const base1 = PAIR ? a.w2 + (int64_t)e * a.stride2 : base0;
+    uint32_t woff[TL::SLOTS];
+    // (recomputed where they are needed: registers are scarcer than the few operations)
+    auto lrow_of = [&](int i) -> int {
+        const int c = tid + GEMM_THREADS * i;
+        const int lr = c < TL::CHUNKS ? c / 17 : 0;
+        return PAIR ? (lr & 63) : lr;
+    };
+    auto piece_of = [&](int i) -> int {
+        const int c = tid + GEMM_THREADS * i;
+        return c < TL::CHUNKS ? 16 * (c % 17) : 0;
+    };
+    auto aim = [&](int block) {   // (a matrix stays below 4 GB)
+#pragma unroll
+        for (int i = 0; i < TL::SLOTS; ++i) {
+            const int row = block * (PAIR ? 64 : TL::ROWS) + lrow_of(i);
+            woff[i] = (uint32_t)(row < a.n ? row : a.n - 1) * (uint32_t)rb + piece_of(i);
+        }
+    };
+    // Every piece is loaded without a condition, so that the loads of a pass leave together and
+    // nothing waits for them before they are stored.  A piece that reaches past the end of its
+    // row is loaded `shift` bytes earlier (always the 16 bytes that end the row) and moved into
+    // place, zeros behind it, when it is stored.
+    auto wshift = [&](int i, int p) -> int {
+        const int over = piece_of(i) + 16 - (rb - Q8_SEG * p);
+        return over < 0 ? 0 : over;
+    };
+    int lrow[NM];
+#pragma unroll
+    for (int j = 0; j < NM; ++j) lrow[j] = PAIR ? j * 64 + wave * 16 + col : wave * (16 * NM) + 16 * j + col;
+    // staging share of this thread: column chunk c8 of token rows tid/32 + 8*j
+    constexpr int NS = 2 * MT;
+    const int c8 = tid & 31, r0 = tid >> 5;
+    // columns 8*c8 .. +7 are columns 8*(c8&3) .. of block c8>>2: two runs of four that belong to
+    // lane groups 2*(c8&1) and 2*(c8&1)+1, in the first or second half of their eight columns
+    const int adst = 64 * (c8 >> 2) + 32 * (c8 & 1) + 8 * ((c8 >> 1) & 1);
+    uint4 st0[NS], st1[NS];
+    u32x4_t wreg[TL::SLOTS];
+    auto request_w = [&](int p) {
+#pragma unroll
+        for (int i = 0; i < TL::SLOTS; ++i) {
+            const uint8_t* base = (PAIR && GEMM_THREADS * i >= 64 * 17) ? base1
+                                  : (PAIR && GEMM_THREADS * (i + 1) > 64 * 17 && tid + GEMM_THREADS * i >= 64 * 17) ? base1 : base0;
+            wreg[i] = ldg_u32x4<4>(base + (woff[i] + (uint32_t)(Q8_SEG * p - wshift(i, p))));
+        }
+    };
+    // the first weights leave before the chunk's activation rows are known
+    aim(rowblock);
+    request_w(0);
+    int arow[NS];
+    bool avalid[NS];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+        const int r = r0 + 8 * j;
+        avalid[j] = r < count;
+        arow[j] = avalid[j] ? (a.gather ? ldg<int>(a.gather + start + r) : start + r) : 0;
+    }
+    auto request_a = [&](int p) {
+        const int c0 = 256 * p + 8 * c8;
+#pragma unroll
+        for (int j = 0; j < NS; ++j) stage_fetch<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
+    };
+    request_a(0);
+    auto multiply = [&]() {
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            OperandBits af[MT][NA];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < NA; ++t) {
+                    const uint4 v = *(const uint4*)(lds + t * TERM + (16 * mt + col) * GEMM_A_STRIDE + 64 * b + 16 * g);
+                    af[mt][t].u[0] = v.x; af[mt][t].u[1] = v.y; af[mt][t].u[2] = v.z; af[mt][t].u[3] = v.w;
+                }
+#pragma unroll
+            for (int j = 0; j < NM; ++j) {
+                const uint8_t* rp = wt + lrow[j] * Q8_ROW;
+                const uint32_t* dw = (const uint32_t*)rp;
+                const float d = half_bits_to_float(*(const uint16_t*)(rp + 34 * b));
+                uint32_t q0, q1;
+                if (b & 1) {
+                    // codes start on a dword
+                    const int at = (34 * b + 2) / 4;
+                    q0 = dw[at + g];
+                    q1 = dw[at + 4 + g];
+                } else {
+                    const int at = (34 * b) / 4;
+                    q0 = __builtin_amdgcn_alignbit(dw[at + g + 1], dw[at + g], 16);
+                    q1 = __builtin_amdgcn_alignbit(dw[at + g + 5], dw[at + g + 4], 16);
+                }
+                OperandBits bt;
+                q8_codes_to_bf16(q0, bt.u[0], bt.u[1]);
+                q8_codes_to_bf16(q1, bt.u[2], bt.u[3]);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    floatx4 c = floatx4{0.f, 0.f, 0.f, 0.f};
+                    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][0].v, bt.v, c, 0, 0, 0);
+                    if (NA == 2) c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][NA - 1].v, bt.v, c, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[j][mt][i] = fmaf(d, c[i], acc[j][mt][i]);
+                }
+            }
+        }
+    };
+    for (int block = rowblock; block < rowblock + nblocks; ++block) {
+        for (int p = 0; p < passes; ++p) {
+            __syncthreads();   // the previous pass has been multiplied
+            const bool ragged = rb - Q8_SEG * p < Q8_SEG;   // the rows end inside this pass
+#pragma unroll
+            for (int i = 0; i < TL::SLOTS; ++i) {
+                u32x4_t v = wreg[i];
+                if (ragged) {
+                    const int sh = (wshift(i, p) < 16 ? wshift(i, p) : 16) >> 2;   // dwords
+                    const u32x4_t t = v;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const int from = d + sh;
+                        v[d] = from == 0 ? t[0] : from == 1 ? t[1] : from == 2 ? t[2] : from == 3 ? t[3] : 0u;
+                    }
+                }
+                if (tid + GEMM_THREADS * i < TL::CHUNKS) *(uint4*)(wt + 16 * (tid + GEMM_THREADS * i)) = make_uint4(v[0], v[1], v[2], v[3]);
+            }
+            const bool cols_live = 256 * p + 8 * c8 < a.k;
+#pragma unroll
+            for (int j = 0; j < NS; ++j) {
+                uint4 hi, lo;
+                stage_terms<AKIND>(st0[j], st1[j], hi, lo);
+                if (!(avalid[j] && cols_live)) hi = lo = make_uint4(0, 0, 0, 0);
+                uint8_t* dst = lds + (r0 + 8 * j) * GEMM_A_STRIDE + adst;
+                *(uint2*)dst = make_uint2(hi.x, hi.y);
+                *(uint2*)(dst + 16) = make_uint2(hi.z, hi.w);
+                if (NA == 2) {
+                    *(uint2*)(dst + TERM) = make_uint2(lo.x, lo.y);
+                    *(uint2*)(dst + TERM + 16) = make_uint2(lo.z, lo.w);
+                }
+            }
+            __syncthreads();
+            if (p + 1 < passes) {
+                request_w(p + 1);
+                request_a(p + 1);
+            } else if (block + 1 < rowblock + nblocks) {
+                aim(block + 1);
+                request_w(0);
+                request_a(0);
+            }
+            multiply();
+        }
+        emit(block);
+#pragma unroll
+        for (int j = 0; j < NM; ++j)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+}
+
 // One chunk (expert e, sorted positions start .. start+count) x this workgroup's rows.
 // NM matrices per wave: the gate and up rows of the same index (PAIR, NM == 2) or NM tiles of
-// 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows.
+// 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows, and `nblocks` of them from there on
+// are this workgroup's (the Q8_0 loop can walk several; the launchers give it one, which measured
+// faster than two or four on the 512-expert step).
 // With SOLO (one token tile, long rows) the four waves share the same 16 * NM rows and split K:
 // wave w walks its quarter of the passes, stages its own activations in its own part of the
 // LDS tile without waiting for the others, and the partial sums meet in LDS at the end.  A
 // matrix with few rows and many columns then has four times as many, four times shorter,
 // work items.
 template <int FMT, int AKIND, bool PAIR, int NM, int MT, bool SOLO>
-__device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds) {
+__device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, int rowblock, int nblocks, uint8_t* lds) {
     static_assert(!PAIR || NM == 2, "a pair is two matrices");
     static_assert(!SOLO || (MT == 1 && !PAIR), "a wave stages one token tile on its own");
     using U = Unit64<FMT>;
@@ -115,6 +349,50 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
     for (int j = 0; j < NM; ++j)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // lane (col, g) holds outputs of tokens 16*mt + 4*g + i, row index col of each matrix
+    auto emit = [&](int block) {
+        int rows[NM];
+        if (PAIR) rows[0] = rows[NM - 1] = block * 64 + wave * 16 + col;
+        else {
+#pragma unroll
+            for (int j = 0; j < NM; ++j) rows[j] = SOLO ? block * (16 * NM) + 16 * j + col : block * (64 * NM) + wave * (16 * NM) + 16 * j + col;
+        }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tk = 16 * mt + 4 * g + i;
+            if (tk >= count) continue;
+            const size_t pos = (size_t)(start + tk);
+            if (PAIR) {
+                if (rows[0] < a.n) {
+                    // SwiGLU, left as two bf16 terms for the down step's A operand when a second array is given
+                    const float v = silu_mul(acc[0][mt][i], acc[NM - 1][mt][i]);
+                    if (a.out1) {
+                        const uint16_t hi = float_to_bf16_bits(v);
+                        const uint16_t lo = float_to_bf16_bits(v - __uint_as_float((uint32_t)hi << 16));
+                        ((uint16_t*)a.out0)[pos * a.n + rows[0]] = hi;
+                        ((uint16_t*)a.out1)[pos * a.n + rows[0]] = lo;
+                    } else {
+                        store_out(a.out0, a.out_dt, pos * a.n + rows[0], v);  // a caller's SwiGLU output
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NM; ++j) {
+                    if (rows[j] >= a.n) continue;
+                    const float v = acc[j][mt][i];
+                    // the routed product is rounded on its own, as the reference stores it
+                    if (a.scale) ((float*)a.out0)[pos * a.n + rows[j]] = mul_unfused(v, a.scale[pos]);
+                    else store_out(a.out0, a.out_dt, pos * a.n + rows[j], v);
+                }
+            }
+        }
+    };
+    if constexpr (FMT == QMOE_FMT_Q8_0 && !SOLO) {
+        q8_tile_loop<AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, nblocks, lds, acc, emit);
+        return;
+    } else {
     // staging share of this thread: column chunk c8 of token rows tid/32 + 8*j (of the wave's
     // own copy: rows lane/32 + 2*j)
     constexpr int NS = SOLO ? 8 : 2 * MT;
@@ -139,13 +417,18 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
 #pragma unroll
         for (int j = 0; j < NM; ++j) U::load_w(rp[j], u, raw[j]);
 #pragma unroll
-        for (int j = 0; j < NS; ++j) stage_load<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
+        for (int j = 0; j < NS; ++j) stage_fetch<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
     }
     for (int p = p_begin; p < passes; ++p) {
         // the previous pass has been multiplied (LDS operations of one wave stay in order)
         if (SOLO) __builtin_amdgcn_wave_barrier(); else __syncthreads();
 #pragma unroll
-        for (int j = 0; j < NS; ++j) stage_store<AKIND, TERM>(st0[j], st1[j], lds + (r0 + RSTEP * j) * GEMM_A_STRIDE + 16 * c8);
+        for (int j = 0; j < NS; ++j) {
+            // (a position outside the chunk or the row was fetched from a valid place: zeros instead)
+            const bool live = avalid[j] && 256 * p + 8 * c8 < a.k;
+            const uint4 zero = make_uint4(0, 0, 0, 0);
+            stage_store<AKIND, TERM>(live ? st0[j] : zero, live ? st1[j] : zero, lds + (r0 + RSTEP * j) * GEMM_A_STRIDE + 16 * c8);
+        }
         if (SOLO) __builtin_amdgcn_wave_barrier(); else __syncthreads();
         const int unit = 4 * p + g;
         const bool live = unit < units;
@@ -154,7 +437,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
         if (p + 1 < passes) {
             const int c0 = 256 * (p + 1) + 8 * c8;
 #pragma unroll
-            for (int j = 0; j < NS; ++j) stage_load<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
+            for (int j = 0; j < NS; ++j) stage_fetch<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j] && c0 < a.k);
         }
         // a unit past the end of the row multiplies as zeros: all-zero bytes decode to 0.0 in
         // every format (zero scales)
@@ -208,6 +491,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
             if (p + 1 < passes) U::load_w(rp[j], un, raw[j]);
         }
     }
+    }
     if (SOLO) {
         // partial sums of the four K ranges: every wave leaves its own in its own LDS part
         floatx4* mine = (floatx4*)lds;
@@ -224,44 +508,24 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
             for (int i = 0; i < 4; ++i) acc[j][0][i] = (acc[j][0][i] + b[i]) + (c[i] + d[i]);
         }
     }
-    // lane (col, g) holds outputs of tokens 16*mt + 4*g + i, row index col of each matrix
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int tk = 16 * mt + 4 * g + i;
-            if (tk >= count) continue;
-            const size_t pos = (size_t)(start + tk);
-            if (PAIR) {
-                if (rows[0] < a.n) {
-                    // SwiGLU, left as two bf16 terms for the down step's A operand when a second array is given
-                    const float v = silu_mul(acc[0][mt][i], acc[NM - 1][mt][i]);
-                    if (a.out1) {
-                        const uint16_t hi = float_to_bf16_bits(v);
-                        const uint16_t lo = float_to_bf16_bits(v - __uint_as_float((uint32_t)hi << 16));
-                        ((uint16_t*)a.out0)[pos * a.n + rows[0]] = hi;
-                        ((uint16_t*)a.out1)[pos * a.n + rows[0]] = lo;
-                    } else {
-                        store_out(a.out0, a.out_dt, pos * a.n + rows[0], v);  // a caller's SwiGLU output
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < NM; ++j) {
-                    if (rows[j] >= a.n) continue;
-                    const float v = acc[j][mt][i];
-                    // the routed product is rounded on its own, as the reference stores it
-                    if (a.scale) ((float*)a.out0)[pos * a.n + rows[j]] = mul_unfused(v, a.scale[pos]);
-                    else store_out(a.out0, a.out_dt, pos * a.n + rows[j], v);
-                }
-            }
-        }
+    emit(rowblock);
 }
 
+// Row tiles per wave and workgroups per CU of the grouped kernel.  Q8_0 keeps a workgroup's LDS and
+// registers small enough for three workgroups a CU where it can (bf16 activations: one staged
+// term; plain rows: one row tile per wave): the kernel waits for memory most of the time and
+// a third workgroup fills part of that.
+template <int FMT, int AKIND, bool PAIR> struct GroupedShape {
+    static constexpr int NM = (FMT == QMOE_FMT_Q8_0 && !PAIR) ? QMOE_PLAIN_NM : 2;
+    static constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
+    static constexpr int LDS = NA * GEMM_TERM_BYTES + (FMT == QMOE_FMT_Q8_0 ? Q8Tile<NM>::BYTES : 0);
+    static constexpr int WGS = (FMT == QMOE_FMT_Q8_0 && LDS * 3 <= 160 * 1024) ? QMOE_BF16_WGS : 2;
+};
+
 template <int FMT, int AKIND, bool PAIR>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_kernel(const GemmArgs a) {
-    constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[NA * GEMM_TERM_BYTES];
+__global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)) void tile_gemm_kernel(const GemmArgs a) {
+    using GS = GroupedShape<FMT, AKIND, PAIR>;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[GS::LDS];
     const int c = blockIdx.y;
     int e = 0, start, count;
     if (a.chunk_expert) {
@@ -274,16 +538,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_kernel(const GemmAr
         count = a.dense_tokens - start < GEMM_CHUNK ? a.dense_tokens - start : GEMM_CHUNK;
     }
     if (count <= 0) return;
-    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, 2, 1, false>(a, e, start, count, blockIdx.x, lds);
-    else tile_gemm_chunk<FMT, AKIND, PAIR, 2, 2, false>(a, e, start, count, blockIdx.x, lds);
+    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 1, false>(a, e, start, count, blockIdx.x, 1, lds);
+    else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, blockIdx.x, 1, lds);
 }
 
 // Several dense matrices (y = W x for `tokens` rows of x each) in one launch: blockIdx.x walks
 // the row blocks of all problems, blockIdx.y the token chunks.
 template <int FMT, int AKIND, int NM>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_dense_kernel(const GemmDenseArgs d) {
+__global__ __launch_bounds__(GEMM_THREADS, (FMT == QMOE_FMT_Q8_0 && AKIND == GEMM_A_BF16) ? QMOE_BF16_WGS : 2) void tile_gemm_dense_kernel(const GemmDenseArgs d) {
     constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * NA * GEMM_TERM_BYTES];  // four solo tiles or one shared tile
+    // four solo tiles, or one shared tile (Q8_0: and the weight tile behind it)
+    constexpr int SHARED = NA * GEMM_TERM_BYTES + (FMT == QMOE_FMT_Q8_0 ? Q8Tile<NM>::BYTES : 0);
+    __shared__ __attribute__((aligned(16))) uint8_t lds[SHARED > 2 * NA * GEMM_TERM_BYTES ? SHARED : 2 * NA * GEMM_TERM_BYTES];
     int i = 0;
     while (i + 1 < d.count && (int)blockIdx.x >= d.block_start[i + 1]) ++i;
     const bool ksplit = d.p[i].ksplit != 0;
@@ -300,16 +566,19 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_dense_kernel(const 
     a.out0 = d.p[i].y;
     a.out_dt = d.p[i].ydt;
     const int rowblock = blockIdx.x - d.block_start[i];
-    if (ksplit) tile_gemm_chunk<FMT, AKIND, false, NM, 1, true>(a, 0, start, count, rowblock, lds);
-    else if (count <= 16) tile_gemm_chunk<FMT, AKIND, false, NM, 1, false>(a, 0, start, count, rowblock, lds);
-    else tile_gemm_chunk<FMT, AKIND, false, NM, 2, false>(a, 0, start, count, rowblock, lds);
+    if (ksplit) tile_gemm_chunk<FMT, AKIND, false, NM, 1, true>(a, 0, start, count, rowblock, 1, lds);
+    else if (count <= 16) tile_gemm_chunk<FMT, AKIND, false, NM, 1, false>(a, 0, start, count, rowblock, 1, lds);
+    else tile_gemm_chunk<FMT, AKIND, false, NM, 2, false>(a, 0, start, count, rowblock, 1, lds);
 }
 
 // ---- host side ------------------------------------------------------------------------------------
+int stream_grid();
+
 bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const void* a0, int a_kind, int64_t a_stride) {
     if (!stream_supported(fmt, w, n, k, nullptr, QMOE_DT_F32)) return false;  // unit loads: same format and alignment rules
     const int align = fmt == QMOE_FMT_Q8_0 ? 4 : fmt == QMOE_FMT_Q6_K ? 2 : 16;
     if (stride % align) return false;
+    if (fmt == QMOE_FMT_Q8_0 && (int64_t)n * (k / 32 * 34) >= (1ll << 32)) return false;  // 32-bit offsets within one matrix
     const int esize = a_kind == GEMM_A_F32 ? 4 : 2;
     return (uintptr_t)a0 % 16 == 0 && (a_stride * esize) % 16 == 0;
 }
@@ -326,7 +595,7 @@ static void gemm_launch_f(const GemmArgs& a, int a_kind, dim3 grid, hipStream_t 
 }
 
 int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, hipStream_t s) {
-    const int rows_per_wg = pair ? 64 : 128;
+    const int rows_per_wg = pair ? 64 : fmt == QMOE_FMT_Q8_0 ? 64 * QMOE_PLAIN_NM : 128;
     const dim3 grid((a.n + rows_per_wg - 1) / rows_per_wg, chunks);
 #define QMOE_GEMM_F(F)                                                  \
     if (pair) gemm_launch_f<F, true>(a, a_kind, grid, s);               \
@@ -352,8 +621,6 @@ static void gemm_dense_f(const GemmDenseArgs& d, int a_kind, dim3 grid, hipStrea
     }
 }
 
-int stream_grid();
-
 // Row blocks of 128 rows when that still fills the chip, else of 64.
 int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     const int chunks = (d.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
@@ -361,7 +628,10 @@ int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     for (int i = 0; i < d.count; ++i) blocks128 += (d.p[i].n + 127) / 128;
     // two row tiles per wave only where the registers hold them without spilling
     const bool roomy = fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_BF16;
-    const int nm = roomy && blocks128 * chunks >= stream_grid() ? 2 : 1;
+    // (Q8_0, whose workgroup keeps a weight tile in flight: two row tiles already where they fill
+    // half the chip -- more bytes on their way per CU outweigh the idle places)
+    const int enough = fmt == QMOE_FMT_Q8_0 ? stream_grid() / 2 : stream_grid();
+    const int nm = roomy && blocks128 * chunks >= enough ? 2 : 1;
     // rows of 8192 columns and more are shared by the four waves (K split), 16 tokens a chunk
     int at = 0, ychunks = chunks;
     for (int i = 0; i < d.count; ++i) {

@@ -86,6 +86,25 @@ def test_linear_low_precision_activations(cuda, dtype, tol, fmt):
     assert rel_l2(got.float().cpu().numpy(), want) <= (5e-3 if dtype == torch.bfloat16 else 1e-3)
 
 
+@pytest.mark.parametrize("shape", [(70, 320), (130, 1408), (64, 64), (200, 2112), (1, 4096)])
+@pytest.mark.parametrize("tokens,dtype", [(3, "f32"), (17, "f32"), (40, "bf16"), (33, "f16")])
+def test_q8_0_token_batches_ragged_rows(cuda, shape, tokens, dtype):
+    """Q8_0 token batches take weight tiles of 64 or 128 rows x 256 columns through LDS: rows whose
+    width ends inside a tile (320, 1408, 64, 2112 columns), row counts that end inside a tile, and
+    a last row that ends the allocation, so nothing may be read behind it."""
+    announce("linear q8_0 ragged", shape, tokens, dtype)
+    w = synthetic.packed_weight("Q8_0", shape, 311)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    x = torch.from_numpy(synthetic.activations((tokens, shape[1]), 312)).to(tdt)
+    want = R.linear(x.float().numpy(), *triple(w))
+    got = quantized_linear(x.to(cuda), upload(w, cuda))
+    assert got.dtype == tdt and got.shape == (tokens, shape[0])
+    tol = {"f32": 2e-5, "f16": 1e-3, "bf16": 5e-3}[dtype]   # fp16 / bf16: the one rounding of the output
+    assert rel_l2(got.float().cpu().numpy(), want) <= tol
+    if dtype == "f32":
+        assert tol <= REL_L2
+
+
 def test_linear_three_dimensional_input_and_shape_errors(cuda):
     w = upload(synthetic.packed_weight("Q4_K", (7, 512), 1), cuda)
     x = torch.from_numpy(synthetic.activations((2, 3, 512), 2)).to(cuda)
