@@ -306,6 +306,184 @@ __device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start
     }
 }
 
+// ---- Q4_K / Q5_K: the same scheme with the 4- and 5-bit codes as the operand ----------------------
+// w = (d * sc) * q - dmin * m for the 32 columns of a group, so with S = the sum of the group's
+// activations   sum_k w x = (d * sc) * sum_k q x  -  (dmin * m) * S :
+// one MFMA per group and activation term over the codes (exact in bf16), two FMAs per output.
+// A pass is one 256-column block of every row (144 / 176 bytes, 9 / 11 pieces of 16 bytes, rows
+// in LDS as they lie in memory); S comes from the activation staging, one value per token and
+// group.  Lane group g takes columns 4g..4g+3 and 16+4g..16+4g+3 of a group as for Q8_0: the
+// nibbles of one dword each, and (Q5_K) bit `group` of the bytes of one dword of the high plane.
+template <int FMT, int NM> struct K45Tile {
+    static constexpr int SEG = FMT == QMOE_FMT_Q5_K ? 176 : 144;
+    static constexpr int QS = FMT == QMOE_FMT_Q5_K ? 48 : 16;
+    static constexpr int PIECES = SEG / 16;
+    static constexpr int ROWS = 64 * NM, CHUNKS = ROWS * PIECES, SLOTS = (CHUNKS + GEMM_THREADS - 1) / GEMM_THREADS;
+    static constexpr int SUMS = 8 * GEMM_CHUNK * 4;          // S[group][token], fp32
+    static constexpr int BYTES = ROWS * SEG + SUMS;
+};
+
+// four unsigned byte codes -> four bf16 (exact)
+__device__ __forceinline__ void byte_codes_to_bf16(uint32_t q, uint32_t& lo2, uint32_t& hi2) {
+    const float f0 = (float)(q & 0xFFu), f1 = (float)((q >> 8) & 0xFFu), f2 = (float)((q >> 16) & 0xFFu), f3 = (float)(q >> 24);
+    lo2 = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+    hi2 = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+}
+
+// sum of the eight staged columns as the GEMM sees them (the value of hi + lo)
+template <int AKIND>
+__device__ __forceinline__ float stage_sum(const uint4 r0, const uint4 r1) {
+    auto two = [](uint32_t w) { return __uint_as_float(w << 16) + __uint_as_float(w & 0xFFFF0000u); };
+    if (AKIND == GEMM_A_F32) {
+        return ((__uint_as_float(r0.x) + __uint_as_float(r0.y)) + (__uint_as_float(r0.z) + __uint_as_float(r0.w))) +
+               ((__uint_as_float(r1.x) + __uint_as_float(r1.y)) + (__uint_as_float(r1.z) + __uint_as_float(r1.w)));
+    } else if (AKIND == GEMM_A_F16) {
+        auto h2 = [](uint32_t w) { return half_bits_to_float(w & 0xFFFFu) + half_bits_to_float(w >> 16); };
+        return (h2(r0.x) + h2(r0.y)) + (h2(r0.z) + h2(r0.w));
+    } else if (AKIND == GEMM_A_PAIR) {
+        return ((two(r0.x) + two(r0.y)) + (two(r0.z) + two(r0.w))) + ((two(r1.x) + two(r1.y)) + (two(r1.z) + two(r1.w)));
+    } else {
+        return (two(r0.x) + two(r0.y)) + (two(r0.z) + two(r0.w));
+    }
+}
+
+template <int FMT, int AKIND, bool PAIR, int NM, int MT, class Emit>
+__device__ __forceinline__ void k45_tile_loop(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds,
+                                              floatx4 (&acc)[NM][MT], Emit emit) {
+    constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
+    constexpr int TERM = GEMM_TERM_BYTES;
+    using TL = K45Tile<FMT, NM>;
+    uint8_t* wt = lds + NA * GEMM_TERM_BYTES;
+    float* sums = (float*)(wt + TL::ROWS * TL::SEG);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 15, g = lane >> 4;
+    const int passes = a.k >> 8;
+    const int rb = passes * TL::SEG;
+    const uint8_t* const base0 = a.w + (int64_t)e * a.stride;
+    const uint8_t* const base1 = PAIR ? a.w2 + (int64_t)e * a.stride2 : base0;
+    // this thread's 16-byte pieces of the weight tile: piece tid + 256*i lies 16 bytes a piece in LDS
+    uint32_t woff[TL::SLOTS];
+#pragma unroll
+    for (int i = 0; i < TL::SLOTS; ++i) {
+        const int c = tid + GEMM_THREADS * i;
+        const int lr = c < TL::CHUNKS ? c / TL::PIECES : 0;
+        const int piece = c < TL::CHUNKS ? c % TL::PIECES : 0;
+        const int row = PAIR ? rowblock * 64 + (lr & 63) : rowblock * TL::ROWS + lr;
+        woff[i] = (uint32_t)(row < a.n ? row : a.n - 1) * (uint32_t)rb + 16 * piece;   // (a matrix stays below 4 GB)
+    }
+    int lrow[NM];
+#pragma unroll
+    for (int j = 0; j < NM; ++j) lrow[j] = PAIR ? j * 64 + wave * 16 + col : wave * (16 * NM) + 16 * j + col;
+    constexpr int NS = 2 * MT;
+    const int c8 = tid & 31, r0 = tid >> 5;
+    const int adst = 64 * (c8 >> 2) + 32 * (c8 & 1) + 8 * ((c8 >> 1) & 1);
+    uint4 st0[NS], st1[NS];
+    u32x4_t wreg[TL::SLOTS];
+    auto request_w = [&](int p) {
+#pragma unroll
+        for (int i = 0; i < TL::SLOTS; ++i) {
+            constexpr int HALF = 64 * TL::PIECES;   // pieces of the first matrix of a pair
+            const uint8_t* base = (PAIR && GEMM_THREADS * i >= HALF) ? base1
+                                  : (PAIR && GEMM_THREADS * (i + 1) > HALF && tid + GEMM_THREADS * i >= HALF) ? base1 : base0;
+            wreg[i] = ldg_u32x4<16>(base + (woff[i] + (uint32_t)(TL::SEG * p)));
+        }
+    };
+    request_w(0);
+    int arow[NS];
+    bool avalid[NS];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+        const int r = r0 + 8 * j;
+        avalid[j] = r < count;
+        arow[j] = avalid[j] ? (a.gather ? ldg<int>(a.gather + start + r) : start + r) : 0;
+    }
+    auto request_a = [&](int p) {
+        const int c0 = 256 * p + 8 * c8;
+#pragma unroll
+        for (int j = 0; j < NS; ++j) stage_fetch<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j]);
+    };
+    request_a(0);
+    for (int p = 0; p < passes; ++p) {
+        __syncthreads();   // the previous pass has been multiplied
+#pragma unroll
+        for (int i = 0; i < TL::SLOTS; ++i)
+            if (tid + GEMM_THREADS * i < TL::CHUNKS)
+                *(uint4*)(wt + 16 * (tid + GEMM_THREADS * i)) = make_uint4(wreg[i][0], wreg[i][1], wreg[i][2], wreg[i][3]);
+#pragma unroll
+        for (int j = 0; j < NS; ++j) {
+            uint4 hi, lo;
+            stage_terms<AKIND>(st0[j], st1[j], hi, lo);
+            float part = stage_sum<AKIND>(st0[j], st1[j]);
+            if (!avalid[j]) { hi = lo = make_uint4(0, 0, 0, 0); part = 0.f; }
+            uint8_t* dst = lds + (r0 + 8 * j) * GEMM_A_STRIDE + adst;
+            *(uint2*)dst = make_uint2(hi.x, hi.y);
+            *(uint2*)(dst + 16) = make_uint2(hi.z, hi.w);
+            if (NA == 2) {
+                *(uint2*)(dst + TERM) = make_uint2(lo.x, lo.y);
+                *(uint2*)(dst + TERM + 16) = make_uint2(lo.z, lo.w);
+            }
+            // the four threads c8 = 4G .. 4G+3 hold the 32 columns of group G of this token
+            part += __shfl_xor(part, 1, 64);
+            part += __shfl_xor(part, 2, 64);
+            if ((c8 & 3) == 0) sums[(c8 >> 2) * GEMM_CHUNK + r0 + 8 * j] = part;
+        }
+        __syncthreads();
+        if (p + 1 < passes) {
+            request_w(p + 1);
+            request_a(p + 1);
+        }
+        // d, dmin and the packed scales of this lane's rows
+        float dd[NM], dm[NM];
+        uint32_t s0[NM], s1[NM], s2[NM];
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            const uint4 h = *(const uint4*)(wt + lrow[j] * TL::SEG);
+            dd[j] = half_bits_to_float(h.x & 0xFFFFu);
+            dm[j] = half_bits_to_float(h.x >> 16);
+            s0[j] = h.y; s1[j] = h.z; s2[j] = h.w;
+        }
+#pragma unroll
+        for (int G = 0; G < 8; ++G) {
+            OperandBits af[MT][NA];
+            floatx4 sx[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                for (int t = 0; t < NA; ++t) {
+                    const uint4 v = *(const uint4*)(lds + t * TERM + (16 * mt + col) * GEMM_A_STRIDE + 64 * G + 16 * g);
+                    af[mt][t].u[0] = v.x; af[mt][t].u[1] = v.y; af[mt][t].u[2] = v.z; af[mt][t].u[3] = v.w;
+                }
+                sx[mt] = *(const floatx4*)(sums + G * GEMM_CHUNK + 16 * mt + 4 * g);
+            }
+#pragma unroll
+            for (int j = 0; j < NM; ++j) {
+                const uint32_t* dw = (const uint32_t*)(wt + lrow[j] * TL::SEG);
+                uint32_t q0 = (dw[TL::QS / 4 + 8 * (G >> 1) + g] >> (4 * (G & 1))) & 0x0F0F0F0Fu;
+                uint32_t q1 = (dw[TL::QS / 4 + 8 * (G >> 1) + 4 + g] >> (4 * (G & 1))) & 0x0F0F0F0Fu;
+                if (FMT == QMOE_FMT_Q5_K) {
+                    q0 |= ((dw[4 + g] >> G) & 0x01010101u) << 4;
+                    q1 |= ((dw[8 + g] >> G) & 0x01010101u) << 4;
+                }
+                OperandBits bt;
+                byte_codes_to_bf16(q0, bt.u[0], bt.u[1]);
+                byte_codes_to_bf16(q1, bt.u[2], bt.u[3]);
+                uint32_t sc, mn;
+                kquant_scale_min(s0[j], s1[j], s2[j], G, sc, mn);
+                const float scale = dd[j] * (float)sc, floor_ = dm[j] * (float)mn;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    floatx4 c = floatx4{0.f, 0.f, 0.f, 0.f};
+                    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][0].v, bt.v, c, 0, 0, 0);
+                    if (NA == 2) c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt][NA - 1].v, bt.v, c, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[j][mt][i] = fmaf(-floor_, sx[mt][i], fmaf(scale, c[i], acc[j][mt][i]));
+                }
+            }
+        }
+    }
+    emit(rowblock);
+}
+
 // One chunk (expert e, sorted positions start .. start+count) x this workgroup's rows.
 // NM matrices per wave: the gate and up rows of the same index (PAIR, NM == 2) or NM tiles of
 // 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows, and `nblocks` of them from there on
@@ -391,6 +569,9 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
     };
     if constexpr (FMT == QMOE_FMT_Q8_0 && !SOLO) {
         q8_tile_loop<AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, nblocks, lds, acc, emit);
+        return;
+    } else if constexpr ((FMT == QMOE_FMT_Q4_K || FMT == QMOE_FMT_Q5_K) && !SOLO) {
+        k45_tile_loop<FMT, AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, lds, acc, emit);
         return;
     } else {
     // staging share of this thread: column chunk c8 of token rows tid/32 + 8*j (of the wave's
@@ -515,11 +696,15 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
 // registers small enough for three workgroups a CU where it can (bf16 activations: one staged
 // term; plain rows: one row tile per wave): the kernel waits for memory most of the time and
 // a third workgroup fills part of that.
+template <int FMT, int NM> struct WeightTile {
+    static constexpr int BYTES = FMT == QMOE_FMT_Q8_0 ? Q8Tile<NM>::BYTES
+                                 : (FMT == QMOE_FMT_Q4_K || FMT == QMOE_FMT_Q5_K) ? K45Tile<FMT, NM>::BYTES : 0;
+};
 template <int FMT, int AKIND, bool PAIR> struct GroupedShape {
     static constexpr int NM = (FMT == QMOE_FMT_Q8_0 && !PAIR) ? QMOE_PLAIN_NM : 2;
     static constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
-    static constexpr int LDS = NA * GEMM_TERM_BYTES + (FMT == QMOE_FMT_Q8_0 ? Q8Tile<NM>::BYTES : 0);
-    static constexpr int WGS = (FMT == QMOE_FMT_Q8_0 && LDS * 3 <= 160 * 1024) ? QMOE_BF16_WGS : 2;
+    static constexpr int LDS = NA * GEMM_TERM_BYTES + WeightTile<FMT, NM>::BYTES;
+    static constexpr int WGS = (WeightTile<FMT, NM>::BYTES != 0 && LDS * 3 <= 160 * 1024) ? QMOE_BF16_WGS : 2;
 };
 
 template <int FMT, int AKIND, bool PAIR>
@@ -548,7 +733,7 @@ template <int FMT, int AKIND, int NM>
 __global__ __launch_bounds__(GEMM_THREADS, (FMT == QMOE_FMT_Q8_0 && AKIND == GEMM_A_BF16) ? QMOE_BF16_WGS : 2) void tile_gemm_dense_kernel(const GemmDenseArgs d) {
     constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
     // four solo tiles, or one shared tile (Q8_0: and the weight tile behind it)
-    constexpr int SHARED = NA * GEMM_TERM_BYTES + (FMT == QMOE_FMT_Q8_0 ? Q8Tile<NM>::BYTES : 0);
+    constexpr int SHARED = NA * GEMM_TERM_BYTES + WeightTile<FMT, NM>::BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t lds[SHARED > 2 * NA * GEMM_TERM_BYTES ? SHARED : 2 * NA * GEMM_TERM_BYTES];
     int i = 0;
     while (i + 1 < d.count && (int)blockIdx.x >= d.block_start[i + 1]) ++i;
@@ -578,7 +763,8 @@ bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const 
     if (!stream_supported(fmt, w, n, k, nullptr, QMOE_DT_F32)) return false;  // unit loads: same format and alignment rules
     const int align = fmt == QMOE_FMT_Q8_0 ? 4 : fmt == QMOE_FMT_Q6_K ? 2 : 16;
     if (stride % align) return false;
-    if (fmt == QMOE_FMT_Q8_0 && (int64_t)n * (k / 32 * 34) >= (1ll << 32)) return false;  // 32-bit offsets within one matrix
+    // (the tile loops address a matrix with 32-bit offsets)
+    if ((fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_Q5_K) && (int64_t)n * row_bytes(fmt, k) >= (1ll << 32)) return false;
     const int esize = a_kind == GEMM_A_F32 ? 4 : 2;
     return (uintptr_t)a0 % 16 == 0 && (a_stride * esize) % 16 == 0;
 }
@@ -627,10 +813,11 @@ int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     int blocks128 = 0;
     for (int i = 0; i < d.count; ++i) blocks128 += (d.p[i].n + 127) / 128;
     // two row tiles per wave only where the registers hold them without spilling
-    const bool roomy = fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_BF16;
-    // (Q8_0, whose workgroup keeps a weight tile in flight: two row tiles already where they fill
-    // half the chip -- more bytes on their way per CU outweigh the idle places)
-    const int enough = fmt == QMOE_FMT_Q8_0 ? stream_grid() / 2 : stream_grid();
+    const bool tiled = fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_Q5_K;
+    const bool roomy = tiled || fmt == QMOE_FMT_BF16;
+    // (the formats whose workgroup keeps a weight tile in flight: two row tiles already where they
+    // fill half the chip -- more bytes on their way per CU outweigh the idle places)
+    const int enough = tiled ? stream_grid() / 2 : stream_grid();
     const int nm = roomy && blocks128 * chunks >= enough ? 2 : 1;
     // rows of 8192 columns and more are shared by the four waves (K split), 16 tokens a chunk
     int at = 0, ychunks = chunks;
