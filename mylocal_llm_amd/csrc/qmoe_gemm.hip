@@ -484,6 +484,154 @@ __device__ __forceinline__ void k45_tile_loop(const GemmArgs& a, int e, int star
     emit(rowblock);
 }
 
+// ---- Q6_K: 6-bit codes as the operand, 16 columns a scale --------------------------------------
+// w = (d * sc) * (q - 32) for the 16 columns of a group:  sum_k w x = (d * sc) * (sum_k q x - 32 S).
+// One v_mfma_f32_16x16x16_bf16 per group and activation term (lane group g multiplies columns
+// 4g..4g+3 of the group: the nibbles of one dword and two bits of the bytes of one dword of the
+// high plane), activations staged in their natural order.  The 210-byte blocks are only 2-byte
+// aligned in memory: a row's block goes to LDS as 13 pieces of 16 bytes plus its scale `d`,
+// rows 240 bytes apart (the 16 rows of a fragment then start in 16 different bank groups).
+template <int NM> struct Q6Tile {
+    static constexpr int SEG = 210, ROW = 240, PIECES = 13;
+    static constexpr int ROWS = 64 * NM, CHUNKS = ROWS * PIECES, SLOTS = (CHUNKS + GEMM_THREADS - 1) / GEMM_THREADS;
+    static constexpr int SUMS = 16 * GEMM_CHUNK * 4;          // S[group][token], fp32
+    static constexpr int BYTES = ROWS * ROW + SUMS;
+};
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+
+template <int AKIND, bool PAIR, int NM, int MT, class Emit>
+__device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds,
+                                             floatx4 (&acc)[NM][MT], Emit emit) {
+    constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
+    constexpr int TERM = GEMM_TERM_BYTES;
+    using TL = Q6Tile<NM>;
+    static_assert(TL::ROWS <= GEMM_THREADS, "one thread a row fetches its scale");
+    uint8_t* wt = lds + NA * GEMM_TERM_BYTES;
+    float* sums = (float*)(wt + TL::ROWS * TL::ROW);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 15, g = lane >> 4;
+    const int passes = a.k >> 8;
+    const int rb = passes * TL::SEG;
+    const uint8_t* const base0 = a.w + (int64_t)e * a.stride;
+    const uint8_t* const base1 = PAIR ? a.w2 + (int64_t)e * a.stride2 : base0;
+    auto row_off = [&](int lr) -> uint32_t {   // (a matrix stays below 4 GB)
+        const int row = PAIR ? rowblock * 64 + (lr & 63) : rowblock * TL::ROWS + lr;
+        return (uint32_t)(row < a.n ? row : a.n - 1) * (uint32_t)rb;
+    };
+    uint32_t woff[TL::SLOTS];
+    int wdst[TL::SLOTS];
+#pragma unroll
+    for (int i = 0; i < TL::SLOTS; ++i) {
+        const int c = tid + GEMM_THREADS * i;
+        const int lr = c < TL::CHUNKS ? c / TL::PIECES : 0;
+        const int piece = c < TL::CHUNKS ? c % TL::PIECES : 0;
+        woff[i] = row_off(lr) + 16 * piece;
+        wdst[i] = lr * TL::ROW + 16 * piece;
+    }
+    const int drow = tid < TL::ROWS ? tid : 0;   // the row whose `d` this thread fetches
+    const uint32_t doff = row_off(drow) + 208;
+    const uint8_t* const dbase = (PAIR && drow >= 64) ? base1 : base0;
+    int lrow[NM];
+#pragma unroll
+    for (int j = 0; j < NM; ++j) lrow[j] = PAIR ? j * 64 + wave * 16 + col : wave * (16 * NM) + 16 * j + col;
+    constexpr int NS = 2 * MT;
+    const int c8 = tid & 31, r0 = tid >> 5;
+    uint4 st0[NS], st1[NS];
+    u32x4_t wreg[TL::SLOTS];
+    uint32_t dreg;
+    auto request_w = [&](int p) {
+#pragma unroll
+        for (int i = 0; i < TL::SLOTS; ++i) {
+            constexpr int HALF = 64 * TL::PIECES;   // pieces of the first matrix of a pair
+            const uint8_t* base = (PAIR && GEMM_THREADS * i >= HALF) ? base1
+                                  : (PAIR && GEMM_THREADS * (i + 1) > HALF && tid + GEMM_THREADS * i >= HALF) ? base1 : base0;
+            wreg[i] = ldg_u32x4<2>(base + (woff[i] + (uint32_t)(TL::SEG * p)));
+        }
+        dreg = ld_u16(dbase + (doff + (uint32_t)(TL::SEG * p)));
+    };
+    request_w(0);
+    int arow[NS];
+    bool avalid[NS];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+        const int r = r0 + 8 * j;
+        avalid[j] = r < count;
+        arow[j] = avalid[j] ? (a.gather ? ldg<int>(a.gather + start + r) : start + r) : 0;
+    }
+    auto request_a = [&](int p) {
+        const int c0 = 256 * p + 8 * c8;
+#pragma unroll
+        for (int j = 0; j < NS; ++j) stage_fetch<AKIND>(st0[j], st1[j], a, arow[j], c0, avalid[j]);
+    };
+    request_a(0);
+    for (int p = 0; p < passes; ++p) {
+        __syncthreads();   // the previous pass has been multiplied
+#pragma unroll
+        for (int i = 0; i < TL::SLOTS; ++i)
+            if (tid + GEMM_THREADS * i < TL::CHUNKS) *(uint4*)(wt + wdst[i]) = make_uint4(wreg[i][0], wreg[i][1], wreg[i][2], wreg[i][3]);
+        if (tid < TL::ROWS) *(uint32_t*)(wt + tid * TL::ROW + 208) = dreg;
+#pragma unroll
+        for (int j = 0; j < NS; ++j) {
+            uint4 hi, lo;
+            stage_terms<AKIND>(st0[j], st1[j], hi, lo);
+            float part = stage_sum<AKIND>(st0[j], st1[j]);
+            if (!avalid[j]) { hi = lo = make_uint4(0, 0, 0, 0); part = 0.f; }
+            uint8_t* dst = lds + (r0 + 8 * j) * GEMM_A_STRIDE + 16 * c8;
+            *(uint4*)dst = hi;
+            if (NA == 2) *(uint4*)(dst + TERM) = lo;
+            // the two threads c8 = 2G, 2G+1 hold the 16 columns of group G of this token
+            part += __shfl_xor(part, 1, 64);
+            if ((c8 & 1) == 0) sums[(c8 >> 1) * GEMM_CHUNK + r0 + 8 * j] = part;
+        }
+        __syncthreads();
+        if (p + 1 < passes) {
+            request_w(p + 1);
+            request_a(p + 1);
+        }
+        float dd[NM];
+        uint4 scw[NM];
+#pragma unroll
+        for (int j = 0; j < NM; ++j) {
+            const uint8_t* rp = wt + lrow[j] * TL::ROW;
+            dd[j] = half_bits_to_float(*(const uint16_t*)(rp + 208));
+            scw[j] = *(const uint4*)(rp + 192);
+        }
+#pragma unroll
+        for (int G = 0; G < 16; ++G) {
+            const int h = G >> 3, Q = (G >> 1) & 3, L = G & 1;
+            union { bf16x4 v; uint2 u; } af[MT][NA];
+            floatx4 sx[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                for (int t = 0; t < NA; ++t) af[mt][t].u = *(const uint2*)(lds + t * TERM + (16 * mt + col) * GEMM_A_STRIDE + 32 * G + 8 * g);
+                sx[mt] = *(const floatx4*)(sums + G * GEMM_CHUNK + 16 * mt + 4 * g);
+            }
+#pragma unroll
+            for (int j = 0; j < NM; ++j) {
+                const uint32_t* dw = (const uint32_t*)(wt + lrow[j] * TL::ROW);
+                const uint32_t ql = dw[16 * h + 8 * (Q & 1) + 4 * L + g];
+                const uint32_t qh = dw[32 + 8 * h + 4 * L + g];
+                const uint32_t code = ((ql >> (4 * (Q >> 1))) & 0x0F0F0F0Fu) | (((qh >> (2 * Q)) & 0x03030303u) << 4);
+                union { bf16x4 v; uint2 u; } bt;
+                byte_codes_to_bf16(code, bt.u.x, bt.u.y);
+                const uint32_t sw = (G >> 2) == 0 ? scw[j].x : (G >> 2) == 1 ? scw[j].y : (G >> 2) == 2 ? scw[j].z : scw[j].w;
+                const float scale = dd[j] * (float)(int)(int8_t)((sw >> (8 * (G & 3))) & 0xFFu);
+                const float off = -32.0f * scale;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    floatx4 c = floatx4{0.f, 0.f, 0.f, 0.f};
+                    c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af[mt][0].v, bt.v, c, 0, 0, 0);
+                    if (NA == 2) c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af[mt][NA - 1].v, bt.v, c, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[j][mt][i] = fmaf(off, sx[mt][i], fmaf(scale, c[i], acc[j][mt][i]));
+                }
+            }
+        }
+    }
+    emit(rowblock);
+}
+
 // One chunk (expert e, sorted positions start .. start+count) x this workgroup's rows.
 // NM matrices per wave: the gate and up rows of the same index (PAIR, NM == 2) or NM tiles of
 // 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows, and `nblocks` of them from there on
@@ -572,6 +720,9 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
         return;
     } else if constexpr ((FMT == QMOE_FMT_Q4_K || FMT == QMOE_FMT_Q5_K) && !SOLO) {
         k45_tile_loop<FMT, AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, lds, acc, emit);
+        return;
+    } else if constexpr (FMT == QMOE_FMT_Q6_K && !SOLO) {
+        q6_tile_loop<AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, lds, acc, emit);
         return;
     } else {
     // staging share of this thread: column chunk c8 of token rows tid/32 + 8*j (of the wave's
@@ -698,7 +849,8 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
 // a third workgroup fills part of that.
 template <int FMT, int NM> struct WeightTile {
     static constexpr int BYTES = FMT == QMOE_FMT_Q8_0 ? Q8Tile<NM>::BYTES
-                                 : (FMT == QMOE_FMT_Q4_K || FMT == QMOE_FMT_Q5_K) ? K45Tile<FMT, NM>::BYTES : 0;
+                                 : (FMT == QMOE_FMT_Q4_K || FMT == QMOE_FMT_Q5_K) ? K45Tile<FMT, NM>::BYTES
+                                 : FMT == QMOE_FMT_Q6_K ? Q6Tile<NM>::BYTES : 0;
 };
 template <int FMT, int AKIND, bool PAIR> struct GroupedShape {
     static constexpr int NM = (FMT == QMOE_FMT_Q8_0 && !PAIR) ? QMOE_PLAIN_NM : 2;
@@ -764,7 +916,7 @@ bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const 
     const int align = fmt == QMOE_FMT_Q8_0 ? 4 : fmt == QMOE_FMT_Q6_K ? 2 : 16;
     if (stride % align) return false;
     // (the tile loops address a matrix with 32-bit offsets)
-    if ((fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_Q5_K) && (int64_t)n * row_bytes(fmt, k) >= (1ll << 32)) return false;
+    if (fmt != QMOE_FMT_BF16 && (int64_t)n * row_bytes(fmt, k) >= (1ll << 32)) return false;
     const int esize = a_kind == GEMM_A_F32 ? 4 : 2;
     return (uintptr_t)a0 % 16 == 0 && (a_stride * esize) % 16 == 0;
 }
@@ -813,7 +965,7 @@ int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     int blocks128 = 0;
     for (int i = 0; i < d.count; ++i) blocks128 += (d.p[i].n + 127) / 128;
     // two row tiles per wave only where the registers hold them without spilling
-    const bool tiled = fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_Q5_K;
+    const bool tiled = fmt != QMOE_FMT_BF16;
     const bool roomy = tiled || fmt == QMOE_FMT_BF16;
     // (the formats whose workgroup keeps a weight tile in flight: two row tiles already where they
     // fill half the chip -- more bytes on their way per CU outweigh the idle places)
