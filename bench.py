@@ -368,7 +368,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extras:
         extras = []
-        for fmt, tokens in (("Q6_K", 1), ("Q5_K", 1), ("Q4_K", 1), ("BF16", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16)):
+        for fmt, tokens in (("Q6_K", 1), ("Q5_K", 1), ("Q4_K", 1), ("BF16", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16), ("Q5_K", 16), ("Q4_K", 16)):
             s = LayerStream(torch, lib, fmt, 8, tokens, device)
             w, m = time_steps(torch, s.step, max(3, args.steps // 4), 2)
             n = max(3, args.steps // 4)
@@ -386,8 +386,9 @@ def main():
         for tokens in (1, 4):
             extras.append(moe_decode_extra(torch, lib, device, "Q8_0", tokens, max(8, args.steps), 3, layer_half=True))
             torch.cuda.empty_cache()
-        extras.append(moe_prefill_extra(torch, lib, device, "Q8_0", 512, 6, 2))
-        torch.cuda.empty_cache()
+        for fmt in ("Q8_0", "Q6_K", "Q5_K"):
+            extras.append(moe_prefill_extra(torch, lib, device, fmt, 512, 6, 2))
+            torch.cuda.empty_cache()
         result["extras"] = extras
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
