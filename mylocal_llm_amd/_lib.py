@@ -43,6 +43,8 @@ class MoeArgs(ctypes.Structure):
                 ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P)]
 
 
+ABI_VERSION = 2   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
+
 _SIGNATURES = {
     "qmoe_abi_version": ([], _I),
     "qmoe_last_error": ([], ctypes.c_char_p),
@@ -83,7 +85,7 @@ def load():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes
                 fn.restype = restype
-            if lib.qmoe_abi_version() != 2:
+            if lib.qmoe_abi_version() != ABI_VERSION:
                 raise RuntimeError(f"{path}: unexpected ABI version {lib.qmoe_abi_version()}")
             _LIB = lib
         return _LIB

@@ -134,12 +134,12 @@ __device__ __forceinline__ void q8_codes_to_bf16(uint32_t q, uint32_t& lo2, uint
     hi2 = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
 }
 
-// The workgroup walks `nblocks` row blocks from `rowblock` on for the same chunk: the weights of
-// the next pass are requested while the current one is multiplied, across row blocks as well, so
-// the wait for the first bytes is paid once per workgroup; emit(block) stores a finished block.
+// emit(rowblock) stores the finished block.  (A workgroup walking two or four row blocks of its
+// chunk with the prefetch carried across measured slower on the 512-expert step: fewer, longer
+// workgroups.)
 template <int AKIND, bool PAIR, int NM, int MT, class Emit>
-__device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start, int count, int rowblock, int nblocks,
-                                             uint8_t* lds, floatx4 (&acc)[NM][MT], Emit emit) {
+__device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds,
+                                             floatx4 (&acc)[NM][MT], Emit emit) {
     constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
     constexpr int TERM = GEMM_TERM_BYTES;
     using TL = Q8Tile<NM>;
@@ -163,13 +163,11 @@ __device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start
         const int c = tid + GEMM_THREADS * i;
         return c < TL::CHUNKS ? 16 * (c % 17) : 0;
     };
-    auto aim = [&](int block) {   // (a matrix stays below 4 GB)
 #pragma unroll
-        for (int i = 0; i < TL::SLOTS; ++i) {
-            const int row = block * (PAIR ? 64 : TL::ROWS) + lrow_of(i);
-            woff[i] = (uint32_t)(row < a.n ? row : a.n - 1) * (uint32_t)rb + piece_of(i);
-        }
-    };
+    for (int i = 0; i < TL::SLOTS; ++i) {   // (a matrix stays below 4 GB)
+        const int row = rowblock * (PAIR ? 64 : TL::ROWS) + lrow_of(i);
+        woff[i] = (uint32_t)(row < a.n ? row : a.n - 1) * (uint32_t)rb + piece_of(i);
+    }
     // Every piece is loaded without a condition, so that the loads of a pass leave together and
     // nothing waits for them before they are stored.  A piece that reaches past the end of its
     // row is loaded `shift` bytes earlier (always the 16 bytes that end the row) and moved into
@@ -198,7 +196,6 @@ __device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start
         }
     };
     // the first weights leave before the chunk's activation rows are known
-    aim(rowblock);
     request_w(0);
     int arow[NS];
     bool avalid[NS];
@@ -255,55 +252,45 @@ __device__ __forceinline__ void q8_tile_loop(const GemmArgs& a, int e, int start
             }
         }
     };
-    for (int block = rowblock; block < rowblock + nblocks; ++block) {
-        for (int p = 0; p < passes; ++p) {
-            __syncthreads();   // the previous pass has been multiplied
-            const bool ragged = rb - Q8_SEG * p < Q8_SEG;   // the rows end inside this pass
+    for (int p = 0; p < passes; ++p) {
+        __syncthreads();   // the previous pass has been multiplied
+        const bool ragged = rb - Q8_SEG * p < Q8_SEG;   // the rows end inside this pass
 #pragma unroll
-            for (int i = 0; i < TL::SLOTS; ++i) {
-                u32x4_t v = wreg[i];
-                if (ragged) {
-                    const int sh = (wshift(i, p) < 16 ? wshift(i, p) : 16) >> 2;   // dwords
-                    const u32x4_t t = v;
+        for (int i = 0; i < TL::SLOTS; ++i) {
+            u32x4_t v = wreg[i];
+            if (ragged) {
+                const int sh = (wshift(i, p) < 16 ? wshift(i, p) : 16) >> 2;   // dwords
+                const u32x4_t t = v;
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        const int from = d + sh;
-                        v[d] = from == 0 ? t[0] : from == 1 ? t[1] : from == 2 ? t[2] : from == 3 ? t[3] : 0u;
-                    }
-                }
-                if (tid + GEMM_THREADS * i < TL::CHUNKS) *(uint4*)(wt + 16 * (tid + GEMM_THREADS * i)) = make_uint4(v[0], v[1], v[2], v[3]);
-            }
-            const bool cols_live = 256 * p + 8 * c8 < a.k;
-#pragma unroll
-            for (int j = 0; j < NS; ++j) {
-                uint4 hi, lo;
-                stage_terms<AKIND>(st0[j], st1[j], hi, lo);
-                if (!(avalid[j] && cols_live)) hi = lo = make_uint4(0, 0, 0, 0);
-                uint8_t* dst = lds + (r0 + 8 * j) * GEMM_A_STRIDE + adst;
-                *(uint2*)dst = make_uint2(hi.x, hi.y);
-                *(uint2*)(dst + 16) = make_uint2(hi.z, hi.w);
-                if (NA == 2) {
-                    *(uint2*)(dst + TERM) = make_uint2(lo.x, lo.y);
-                    *(uint2*)(dst + TERM + 16) = make_uint2(lo.z, lo.w);
+                for (int d = 0; d < 4; ++d) {
+                    const int from = d + sh;
+                    v[d] = from == 0 ? t[0] : from == 1 ? t[1] : from == 2 ? t[2] : from == 3 ? t[3] : 0u;
                 }
             }
-            __syncthreads();
-            if (p + 1 < passes) {
-                request_w(p + 1);
-                request_a(p + 1);
-            } else if (block + 1 < rowblock + nblocks) {
-                aim(block + 1);
-                request_w(0);
-                request_a(0);
-            }
-            multiply();
+            if (tid + GEMM_THREADS * i < TL::CHUNKS) *(uint4*)(wt + 16 * (tid + GEMM_THREADS * i)) = make_uint4(v[0], v[1], v[2], v[3]);
         }
-        emit(block);
+        const bool cols_live = 256 * p + 8 * c8 < a.k;
 #pragma unroll
-        for (int j = 0; j < NM; ++j)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[j][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NS; ++j) {
+            uint4 hi, lo;
+            stage_terms<AKIND>(st0[j], st1[j], hi, lo);
+            if (!(avalid[j] && cols_live)) hi = lo = make_uint4(0, 0, 0, 0);
+            uint8_t* dst = lds + (r0 + 8 * j) * GEMM_A_STRIDE + adst;
+            *(uint2*)dst = make_uint2(hi.x, hi.y);
+            *(uint2*)(dst + 16) = make_uint2(hi.z, hi.w);
+            if (NA == 2) {
+                *(uint2*)(dst + TERM) = make_uint2(lo.x, lo.y);
+                *(uint2*)(dst + TERM + 16) = make_uint2(lo.z, lo.w);
+            }
+        }
+        __syncthreads();
+        if (p + 1 < passes) {
+            request_w(p + 1);
+            request_a(p + 1);
+        }
+        multiply();
     }
+    emit(rowblock);
 }
 
 // ---- Q4_K / Q5_K: the same scheme with the 4- and 5-bit codes as the operand ----------------------
@@ -634,16 +621,14 @@ __device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start
 
 // One chunk (expert e, sorted positions start .. start+count) x this workgroup's rows.
 // NM matrices per wave: the gate and up rows of the same index (PAIR, NM == 2) or NM tiles of
-// 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows, and `nblocks` of them from there on
-// are this workgroup's (the Q8_0 loop can walk several; the launchers give it one, which measured
-// faster than two or four on the 512-expert step).
+// 16 rows; `rowblock` counts blocks of 64 (pair) or 64 * NM rows.
 // With SOLO (one token tile, long rows) the four waves share the same 16 * NM rows and split K:
 // wave w walks its quarter of the passes, stages its own activations in its own part of the
 // LDS tile without waiting for the others, and the partial sums meet in LDS at the end.  A
 // matrix with few rows and many columns then has four times as many, four times shorter,
 // work items.
 template <int FMT, int AKIND, bool PAIR, int NM, int MT, bool SOLO>
-__device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, int rowblock, int nblocks, uint8_t* lds) {
+__device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds) {
     static_assert(!PAIR || NM == 2, "a pair is two matrices");
     static_assert(!SOLO || (MT == 1 && !PAIR), "a wave stages one token tile on its own");
     using U = Unit64<FMT>;
@@ -716,7 +701,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
         }
     };
     if constexpr (FMT == QMOE_FMT_Q8_0 && !SOLO) {
-        q8_tile_loop<AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, nblocks, lds, acc, emit);
+        q8_tile_loop<AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, lds, acc, emit);
         return;
     } else if constexpr ((FMT == QMOE_FMT_Q4_K || FMT == QMOE_FMT_Q5_K) && !SOLO) {
         k45_tile_loop<FMT, AKIND, PAIR, NM, MT>(a, e, start, count, rowblock, lds, acc, emit);
@@ -875,8 +860,8 @@ __global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)
         count = a.dense_tokens - start < GEMM_CHUNK ? a.dense_tokens - start : GEMM_CHUNK;
     }
     if (count <= 0) return;
-    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 1, false>(a, e, start, count, blockIdx.x, 1, lds);
-    else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, blockIdx.x, 1, lds);
+    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 1, false>(a, e, start, count, blockIdx.x, lds);
+    else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, blockIdx.x, lds);
 }
 
 // Several dense matrices (y = W x for `tokens` rows of x each) in one launch: blockIdx.x walks
@@ -903,9 +888,9 @@ __global__ __launch_bounds__(GEMM_THREADS, (FMT == QMOE_FMT_Q8_0 && AKIND == GEM
     a.out0 = d.p[i].y;
     a.out_dt = d.p[i].ydt;
     const int rowblock = blockIdx.x - d.block_start[i];
-    if (ksplit) tile_gemm_chunk<FMT, AKIND, false, NM, 1, true>(a, 0, start, count, rowblock, 1, lds);
-    else if (count <= 16) tile_gemm_chunk<FMT, AKIND, false, NM, 1, false>(a, 0, start, count, rowblock, 1, lds);
-    else tile_gemm_chunk<FMT, AKIND, false, NM, 2, false>(a, 0, start, count, rowblock, 1, lds);
+    if (ksplit) tile_gemm_chunk<FMT, AKIND, false, NM, 1, true>(a, 0, start, count, rowblock, lds);
+    else if (count <= 16) tile_gemm_chunk<FMT, AKIND, false, NM, 1, false>(a, 0, start, count, rowblock, lds);
+    else tile_gemm_chunk<FMT, AKIND, false, NM, 2, false>(a, 0, start, count, rowblock, lds);
 }
 
 // ---- host side ------------------------------------------------------------------------------------

@@ -75,7 +75,17 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_lib.EXPORTS)
     for name in names:
         assert getattr(lib, name) is not None
-    assert lib.qmoe_abi_version() == 2
+    # the header, the binding and the built library agree on the ABI version
+    with open(os.path.join(ROOT, "include", "qmoe.h")) as fh:
+        declared = int(re.search(r"#define\s+QMOE_ABI_VERSION\s+(\d+)", fh.read()).group(1))
+    assert lib.qmoe_abi_version() == declared == _lib.ABI_VERSION
+
+
+def test_driver_build_entry_checks_the_bound_version():
+    """build() of the driver entry module must not pin a version of its own."""
+    with open(os.path.join(ROOT, "__graft_entry__.py")) as fh:
+        text = fh.read()
+    assert "_lib.ABI_VERSION" in text and not re.search(r"qmoe_abi_version\(\)\s*==\s*\d", text)
 
 
 def test_format_info_matches_table():
