@@ -28,6 +28,9 @@ static constexpr int GEMM_THREADS = 256;
 #ifndef QMOE_BF16_WGS
 #define QMOE_BF16_WGS 3
 #endif
+#ifndef QMOE_SPARSE_DIV
+#define QMOE_SPARSE_DIV 2
+#endif
 #ifndef QMOE_PLAIN_NM
 #define QMOE_PLAIN_NM 1
 #endif
@@ -949,17 +952,19 @@ int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     const int chunks = (d.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
     int blocks128 = 0;
     for (int i = 0; i < d.count; ++i) blocks128 += (d.p[i].n + 127) / 128;
-    // two row tiles per wave only where the registers hold them without spilling
-    const bool tiled = fmt != QMOE_FMT_BF16;
-    const bool roomy = tiled || fmt == QMOE_FMT_BF16;
-    // (the formats whose workgroup keeps a weight tile in flight: two row tiles already where they
-    // fill half the chip -- more bytes on their way per CU outweigh the idle places)
-    const int enough = tiled ? stream_grid() / 2 : stream_grid();
-    const int nm = roomy && blocks128 * chunks >= enough ? 2 : 1;
-    // rows of 8192 columns and more are shared by the four waves (K split), 16 tokens a chunk
+    // The formats whose workgroup keeps a weight tile in flight take two row tiles per wave already
+    // where that fills half the chip: more bytes on their way per CU outweigh the idle places.
+    const int enough = fmt != QMOE_FMT_BF16 ? stream_grid() / 2 : stream_grid();
+    const int nm = blocks128 * chunks >= enough ? 2 : 1;
+    // Rows of 8192 columns and more are shared by the four waves of a workgroup (K split, 16 rows
+    // and 16 tokens a workgroup); so is every matrix of a launch that would not fill half the chip
+    // with 64-row workgroups (a lone attention projection: 64 workgroups walking 16 passes each).
+    int blocks64 = 0;
+    for (int i = 0; i < d.count; ++i) blocks64 += (d.p[i].n + 63) / 64;
+    const bool sparse = (int64_t)blocks64 * chunks < stream_grid() / QMOE_SPARSE_DIV;
     int at = 0, ychunks = chunks;
     for (int i = 0; i < d.count; ++i) {
-        d.p[i].ksplit = d.p[i].k >= 8192;
+        d.p[i].ksplit = d.p[i].k >= 8192 || (sparse && d.p[i].k >= 1024);
         const int rows_per_block = d.p[i].ksplit ? 16 * nm : 64 * nm;
         d.block_start[i] = at;
         at += (d.p[i].n + rows_per_block - 1) / rows_per_block;

@@ -138,12 +138,12 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
         args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, 0, xdt, ydt, 0, 0};
         return stream_launch(args, s);
     }
-    // token batches: the token-tile GEMM when its 64-row blocks fill the chip (or the batch is
-    // beyond the small-batch kernel), else the small-batch kernel with its 16-row tiles
+    // token batches: the token-tile GEMM (it splits K over the waves of a workgroup when the matrix
+    // alone would leave most of the chip idle); the small-batch kernel where the GEMM's alignment
+    // rules do not hold
     const bool tile_ok = tokens >= 2 && gemm_supported(fmt, w, 0, n, k, x, xdt, k);
     const bool small_ok = smallm_supported(fmt, w, n, k, x, xdt, tokens);
-    const long tile_groups = (long)((n + 63) / 64) * ((tokens + GEMM_CHUNK - 1) / GEMM_CHUNK);
-    if (tile_ok && (!small_ok || tile_groups >= stream_grid() / 2)) {
+    if (tile_ok) {
         GemmDenseArgs d{};
         d.count = 1;
         d.tokens = tokens;
