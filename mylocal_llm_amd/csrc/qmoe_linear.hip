@@ -139,10 +139,8 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
         return stream_launch(args, s);
     }
     // token batches: the token-tile GEMM (it splits K over the waves of a workgroup when the matrix
-    // alone would leave most of the chip idle); the small-batch kernel where the GEMM's alignment
-    // rules do not hold
+    // alone would leave most of the chip idle); the general kernel where its rules do not hold
     const bool tile_ok = tokens >= 2 && gemm_supported(fmt, w, 0, n, k, x, xdt, k);
-    const bool small_ok = smallm_supported(fmt, w, n, k, x, xdt, tokens);
     if (tile_ok) {
         GemmDenseArgs d{};
         d.count = 1;
@@ -150,7 +148,6 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
         d.p[0] = GemmDenseProblem{(const uint8_t*)w, x, y, n, k, ydt, 0};
         return gemm_dense_launch(fmt, xdt, d, s);
     }
-    if (small_ok) return smallm_launch(fmt, w, n, k, x, xdt, tokens, y, ydt, s);
     const bool fast = rows_fast(fmt, w, row_bytes(fmt, k), k) && x_fast(x, xdt, k);
     if (xdt == QMOE_DT_F32) launch_linear_mt<QMOE_DT_F32>(w, fmt, n, k, fast, x, tokens, y, ydt, s);
     else if (xdt == QMOE_DT_F16) launch_linear_mt<QMOE_DT_F16>(w, fmt, n, k, fast, x, tokens, y, ydt, s);

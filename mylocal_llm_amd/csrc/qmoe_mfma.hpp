@@ -1,4 +1,4 @@
-// bf16 MFMA operand helpers shared by the small-batch linear and the token-tile GEMM.
+// bf16 MFMA operand helpers of the token-tile GEMM.
 #pragma once
 #include "qmoe_common.hpp"
 

@@ -762,11 +762,6 @@ int stream_launch(StreamArgs& args, hipStream_t s);
 
 int stream_grid();
 
-// ---- small-batch MFMA linear (qmoe_smallm.hip) ------------------------------------------------
-bool smallm_supported(int fmt, const void* w, int n, int k, const void* x, int xdt, int tokens);
-int smallm_launch(int fmt, const void* w, int n, int k, const void* x, int xdt, int tokens, void* y, int ydt,
-                  hipStream_t s);
-
 // ---- decode-time MoE step (qmoe_decode.hip) -----------------------------------------------------
 struct DecodeBuffers {  // workspace regions, all device pointers
     float* weights;
