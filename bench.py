@@ -73,7 +73,7 @@ def device_blocks(torch, fmt, n, k, gen, device):
 class LayerStream:
     """`layers` x 7 packed projections resident in HBM plus activation / output buffers."""
 
-    def __init__(self, torch, lib, fmt, layers, tokens, device, seed=106):
+    def __init__(self, torch, lib, fmt, layers, tokens, device, seed=106, act="f32"):
         from mylocal_llm_amd import _lib
         self.torch, self.lib, self.fmt, self.layers, self.tokens = torch, lib, fmt, layers, tokens
         gen = torch.Generator(device=device)
@@ -83,10 +83,11 @@ class LayerStream:
         xgen.manual_seed(103)
         # one activation buffer per data-flow group: (q, k, v) share the layer input, o reads the
         # attention output, (gate, up) the post-attention state, down the SwiGLU activation
-        self.x = {name: torch.randn((tokens, k), device=device, generator=xgen)
+        tdt, dt_id = {"f32": (torch.float32, 0), "f16": (torch.float16, 1), "bf16": (torch.bfloat16, 2)}[act]
+        self.x = {name: torch.randn((tokens, k), device=device, generator=xgen).to(tdt)
                   for name, k in (("qkv", 4096), ("o", 4096), ("gateup", 4096), ("down", 14336))}
         group = {"q": "qkv", "k": "qkv", "v": "qkv", "o": "o", "gate": "gateup", "up": "gateup", "down": "down"}
-        self.y = [torch.empty((tokens, n), device=device) for _, n, _ in PROJECTIONS]
+        self.y = [torch.empty((tokens, n), device=device, dtype=tdt) for _, n, _ in PROJECTIONS]
         self.bytes_per_layer = sum(weight_bytes(fmt, n, k) for _, n, k in PROJECTIONS)
         fid = _lib.FORMAT_ID[fmt]
         self.batches = []
@@ -95,7 +96,7 @@ class LayerStream:
             for i, (name, n, k) in enumerate(PROJECTIONS):
                 p = arr[i]
                 p.w, p.x, p.y = self.weights[layer][i].data_ptr(), self.x[group[name]].data_ptr(), self.y[i].data_ptr()
-                p.fmt, p.n, p.k, p.tokens, p.x_dtype, p.y_dtype = fid, n, k, tokens, 0, 0
+                p.fmt, p.n, p.k, p.tokens, p.x_dtype, p.y_dtype = fid, n, k, tokens, dt_id, dt_id
             self.batches.append(arr)
         self.launches_per_step = layers  # one batched launch sequence per layer
 
@@ -368,12 +369,14 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extras:
         extras = []
-        for fmt, tokens in (("Q6_K", 1), ("Q5_K", 1), ("Q4_K", 1), ("BF16", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16), ("Q5_K", 16), ("Q4_K", 16)):
-            s = LayerStream(torch, lib, fmt, 8, tokens, device)
+        for fmt, tokens, act in (("Q6_K", 1, "f32"), ("Q5_K", 1, "f32"), ("Q4_K", 1, "f32"), ("BF16", 1, "f32"), ("Q8_0", 4, "f32"),
+                                 ("Q8_0", 16, "f32"), ("Q8_0", 64, "f32"), ("Q6_K", 16, "f32"), ("Q5_K", 16, "f32"), ("Q4_K", 16, "f32"),
+                                 ("Q8_0", 16, "bf16"), ("Q8_0", 64, "bf16"), ("Q5_K", 16, "bf16")):
+            s = LayerStream(torch, lib, fmt, 8, tokens, device, act=act)
             w, m = time_steps(torch, s.step, max(3, args.steps // 4), 2)
             n = max(3, args.steps // 4)
             per_layer = m / n / 8 * 1e-3
-            extras.append({"workload": f"8B projections {fmt} M={tokens} (8 layers)",
+            extras.append({"workload": f"8B projections {fmt} M={tokens} (8 layers)" + ("" if act == "f32" else f", {act} activations"),
                            "GBps": round(s.bytes_per_layer / per_layer / 1e9, 1),
                            "frac_hbm_peak": round(s.bytes_per_layer / per_layer / 1e9 / HBM_PEAK_GBS, 4),
                            "us_per_layer": round(per_layer * 1e6, 2),

@@ -25,21 +25,11 @@
 namespace qmoe {
 
 static constexpr int GEMM_THREADS = 256;
-#ifndef QMOE_BF16_WGS
-#define QMOE_BF16_WGS 3
-#endif
-#ifndef QMOE_SPARSE_DIV
-#define QMOE_SPARSE_DIV 2
-#endif
-#ifndef QMOE_PLAIN_NM
-#define QMOE_PLAIN_NM 1
-#endif
+// measured choices (512-expert step at T = 512 and the 8B layer at 4..64 tokens):
+static constexpr int GEMM_SLIM_WGS = 3;        // workgroups a CU where a kernel's LDS and registers allow a third
+static constexpr int GEMM_Q8_PLAIN_TILES = 1;  // row tiles per wave of the grouped Q8_0 kernel over plain rows
 static constexpr int GEMM_A_STRIDE = 528;                       // bytes of one staged token row
 static constexpr int GEMM_TERM_BYTES = GEMM_CHUNK * GEMM_A_STRIDE;  // one bf16 term of the chunk
-
-template <int AKIND> struct AStage {
-    static constexpr int WORDS = (AKIND == GEMM_A_F32 || AKIND == GEMM_A_PAIR) ? 2 : 1;
-};
 
 // Eight consecutive columns of one activation row, as they lie in memory; a position outside
 // the chunk or the row reads (valid) element 0 instead.  The caller zeroes such a position when
@@ -841,10 +831,10 @@ template <int FMT, int NM> struct WeightTile {
                                  : FMT == QMOE_FMT_Q6_K ? Q6Tile<NM>::BYTES : 0;
 };
 template <int FMT, int AKIND, bool PAIR> struct GroupedShape {
-    static constexpr int NM = (FMT == QMOE_FMT_Q8_0 && !PAIR) ? QMOE_PLAIN_NM : 2;
+    static constexpr int NM = (FMT == QMOE_FMT_Q8_0 && !PAIR) ? GEMM_Q8_PLAIN_TILES : 2;
     static constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
     static constexpr int LDS = NA * GEMM_TERM_BYTES + WeightTile<FMT, NM>::BYTES;
-    static constexpr int WGS = (WeightTile<FMT, NM>::BYTES != 0 && LDS * 3 <= 160 * 1024) ? QMOE_BF16_WGS : 2;
+    static constexpr int WGS = (WeightTile<FMT, NM>::BYTES != 0 && LDS * 3 <= 160 * 1024) ? GEMM_SLIM_WGS : 2;
 };
 
 template <int FMT, int AKIND, bool PAIR>
@@ -870,7 +860,7 @@ __global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)
 // Several dense matrices (y = W x for `tokens` rows of x each) in one launch: blockIdx.x walks
 // the row blocks of all problems, blockIdx.y the token chunks.
 template <int FMT, int AKIND, int NM>
-__global__ __launch_bounds__(GEMM_THREADS, (FMT == QMOE_FMT_Q8_0 && AKIND == GEMM_A_BF16) ? QMOE_BF16_WGS : 2) void tile_gemm_dense_kernel(const GemmDenseArgs d) {
+__global__ __launch_bounds__(GEMM_THREADS, (FMT == QMOE_FMT_Q8_0 && AKIND == GEMM_A_BF16) ? GEMM_SLIM_WGS : 2) void tile_gemm_dense_kernel(const GemmDenseArgs d) {
     constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
     // four solo tiles, or one shared tile (Q8_0: and the weight tile behind it)
     constexpr int SHARED = NA * GEMM_TERM_BYTES + WeightTile<FMT, NM>::BYTES;
@@ -921,7 +911,7 @@ static void gemm_launch_f(const GemmArgs& a, int a_kind, dim3 grid, hipStream_t 
 }
 
 int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, hipStream_t s) {
-    const int rows_per_wg = pair ? 64 : fmt == QMOE_FMT_Q8_0 ? 64 * QMOE_PLAIN_NM : 128;
+    const int rows_per_wg = pair ? 64 : fmt == QMOE_FMT_Q8_0 ? 64 * GEMM_Q8_PLAIN_TILES : 128;
     const dim3 grid((a.n + rows_per_wg - 1) / rows_per_wg, chunks);
 #define QMOE_GEMM_F(F)                                                  \
     if (pair) gemm_launch_f<F, true>(a, a_kind, grid, s);               \
@@ -961,7 +951,7 @@ int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s) {
     // with 64-row workgroups (a lone attention projection: 64 workgroups walking 16 passes each).
     int blocks64 = 0;
     for (int i = 0; i < d.count; ++i) blocks64 += (d.p[i].n + 63) / 64;
-    const bool sparse = (int64_t)blocks64 * chunks < stream_grid() / QMOE_SPARSE_DIV;
+    const bool sparse = (int64_t)blocks64 * chunks < stream_grid() / 2;
     int at = 0, ychunks = chunks;
     for (int i = 0; i < d.count; ++i) {
         d.p[i].ksplit = d.p[i].k >= 8192 || (sparse && d.p[i].k >= 1024);
