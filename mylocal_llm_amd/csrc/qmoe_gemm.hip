@@ -465,7 +465,9 @@ __device__ __forceinline__ void k45_tile_loop(const GemmArgs& a, int e, int star
 }
 
 // ---- Q6_K: 6-bit codes as the operand, 16 columns a scale --------------------------------------
-// w = (d * sc) * (q - 32) for the 16 columns of a group:  sum_k w x = (d * sc) * (sum_k q x - 32 S).
+// w = (d * sc) * (q - 32) for the 16 columns of a group.  With bit 5 of a code flipped and the code
+// shifted up by two, its byte read as an int8 is 4 * (q - 32): that is the operand (exact in
+// bf16), and the group's partial product is scaled by (d * sc) / 4 -- no offset term.
 // One v_mfma_f32_16x16x16_bf16 per group and activation term (lane group g multiplies columns
 // 4g..4g+3 of the group: the nibbles of one dword and two bits of the bytes of one dword of the
 // high plane), activations staged in their natural order.  The 210-byte blocks are only 2-byte
@@ -474,8 +476,7 @@ __device__ __forceinline__ void k45_tile_loop(const GemmArgs& a, int e, int star
 template <int NM> struct Q6Tile {
     static constexpr int SEG = 210, ROW = 240, PIECES = 13;
     static constexpr int ROWS = 64 * NM, CHUNKS = ROWS * PIECES, SLOTS = (CHUNKS + GEMM_THREADS - 1) / GEMM_THREADS;
-    static constexpr int SUMS = 16 * GEMM_CHUNK * 4;          // S[group][token], fp32
-    static constexpr int BYTES = ROWS * ROW + SUMS;
+    static constexpr int BYTES = ROWS * ROW;
 };
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 
@@ -487,7 +488,6 @@ __device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start
     using TL = Q6Tile<NM>;
     static_assert(TL::ROWS <= GEMM_THREADS, "one thread a row fetches its scale");
     uint8_t* wt = lds + NA * GEMM_TERM_BYTES;
-    float* sums = (float*)(wt + TL::ROWS * TL::ROW);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 15, g = lane >> 4;
     const int passes = a.k >> 8;
@@ -554,14 +554,10 @@ __device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start
         for (int j = 0; j < NS; ++j) {
             uint4 hi, lo;
             stage_terms<AKIND>(st0[j], st1[j], hi, lo);
-            float part = stage_sum<AKIND>(st0[j], st1[j]);
-            if (!avalid[j]) { hi = lo = make_uint4(0, 0, 0, 0); part = 0.f; }
+            if (!avalid[j]) hi = lo = make_uint4(0, 0, 0, 0);
             uint8_t* dst = lds + (r0 + 8 * j) * GEMM_A_STRIDE + 16 * c8;
             *(uint4*)dst = hi;
             if (NA == 2) *(uint4*)(dst + TERM) = lo;
-            // the two threads c8 = 2G, 2G+1 hold the 16 columns of group G of this token
-            part += __shfl_xor(part, 1, 64);
-            if ((c8 & 1) == 0) sums[(c8 >> 1) * GEMM_CHUNK + r0 + 8 * j] = part;
         }
         __syncthreads();
         if (p + 1 < passes) {
@@ -580,13 +576,10 @@ __device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start
         for (int G = 0; G < 16; ++G) {
             const int h = G >> 3, Q = (G >> 1) & 3, L = G & 1;
             union { bf16x4 v; uint2 u; } af[MT][NA];
-            floatx4 sx[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int t = 0; t < NA; ++t) af[mt][t].u = *(const uint2*)(lds + t * TERM + (16 * mt + col) * GEMM_A_STRIDE + 32 * G + 8 * g);
-                sx[mt] = *(const floatx4*)(sums + G * GEMM_CHUNK + 16 * mt + 4 * g);
-            }
 #pragma unroll
             for (int j = 0; j < NM; ++j) {
                 const uint32_t* dw = (const uint32_t*)(wt + lrow[j] * TL::ROW);
@@ -594,17 +587,16 @@ __device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start
                 const uint32_t qh = dw[32 + 8 * h + 4 * L + g];
                 const uint32_t code = ((ql >> (4 * (Q >> 1))) & 0x0F0F0F0Fu) | (((qh >> (2 * Q)) & 0x03030303u) << 4);
                 union { bf16x4 v; uint2 u; } bt;
-                byte_codes_to_bf16(code, bt.u.x, bt.u.y);
+                q8_codes_to_bf16((code ^ 0x20202020u) << 2, bt.u.x, bt.u.y);   // bytes <= 63: no carry between them
                 const uint32_t sw = (G >> 2) == 0 ? scw[j].x : (G >> 2) == 1 ? scw[j].y : (G >> 2) == 2 ? scw[j].z : scw[j].w;
-                const float scale = dd[j] * (float)(int)(int8_t)((sw >> (8 * (G & 3))) & 0xFFu);
-                const float off = -32.0f * scale;
+                const float scale = (0.25f * dd[j]) * (float)(int)(int8_t)((sw >> (8 * (G & 3))) & 0xFFu);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     floatx4 c = floatx4{0.f, 0.f, 0.f, 0.f};
                     c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af[mt][0].v, bt.v, c, 0, 0, 0);
                     if (NA == 2) c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af[mt][NA - 1].v, bt.v, c, 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[j][mt][i] = fmaf(off, sx[mt][i], fmaf(scale, c[i], acc[j][mt][i]));
+                    for (int i = 0; i < 4; ++i) acc[j][mt][i] = fmaf(scale, c[i], acc[j][mt][i]);
                 }
             }
         }
