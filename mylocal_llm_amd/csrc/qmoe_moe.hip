@@ -22,7 +22,11 @@ int router_topk_impl(const float* logits, int tokens, int n, int k, float floor_
                      int64_t* ids, hipStream_t s);
 
 static constexpr int PLAN_THREADS = 1024;
-static constexpr int GEMM_MIN_TOKENS = 17;  // fewer tokens take the decode path
+// Up to 16 tokens take the decode path where it applies (it is asked first); shapes outside it
+// (an expert width that is no power-of-two multiple of 128, a shared expert in another format ...)
+// take the token-tile GEMMs at any token count: at 16 tokens an order of magnitude faster than the
+// general kernels.
+static constexpr int GEMM_MIN_TOKENS = 1;
 static constexpr size_t PLAN_LDS_LIMIT = 60 * 1024;
 
 // Block-wide exclusive scan of one int per thread (PLAN_THREADS threads); returns the

@@ -337,6 +337,30 @@ def test_moe_token_batches_ragged_shapes(cuda, fmt, dtype):
     assert rel_l2(out.float().cpu().numpy(), want) <= tol <= REL_L2
 
 
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q5_K"])
+@pytest.mark.parametrize("tokens", [1, 3, 16])
+def test_few_tokens_outside_the_decode_shapes(cuda, fmt, tokens):
+    """Expert widths the decode launches do not cover (768 = 6 x 128 columns; a shared expert in
+    another format than the bank): few tokens then take the token-tile GEMMs, same results."""
+    announce("moe few tokens, other shapes", fmt, tokens)
+    e, d, f, fsh, k = 16, 512, 768, 256, 4
+    gate, up, down, _, gate_vec = make_layer(e, d, f, fsh, (fmt, fmt, fmt), 2100)
+    shared = (synthetic.packed_weight("Q8_0", (fsh, d), 2101), synthetic.packed_weight("Q8_0", (fsh, d), 2102),
+              synthetic.packed_weight("Q6_K", (d, fsh), 2103))
+    scale = np.float32(2.0 if fmt == "Q8_0" else 2.0 ** -6)
+    hidden = synthetic.activations((tokens, d), 31, "bf16") * scale
+    logits = synthetic.router_logits(tokens, e, 33)
+    assert not synthetic.has_topk_ties(logits, k)
+    want, want_w, want_ids = oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    out, w, ids = moe_step(torch.from_numpy(hidden).to(cuda), bank, k, logits=torch.from_numpy(logits).to(cuda),
+                           shared=tuple(upload(x, cuda) for x in shared), shared_gate=torch.from_numpy(gate_vec).to(cuda),
+                           return_routing=True)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=0)
+    assert rel_l2(out.cpu().numpy(), want) <= 2e-5 <= REL_L2
+
+
 @pytest.mark.parametrize("tokens", [2, 7])
 def test_decode_path_with_more_experts_than_the_fused_launch_routes(cuda, tokens):
     """1536 experts: wider than the rows the fused route + gate/up launch keeps in registers, so a
