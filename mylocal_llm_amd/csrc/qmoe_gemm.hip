@@ -849,6 +849,27 @@ __global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)
     else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, blockIdx.x, lds);
 }
 
+// Plain rows over hi/lo activations, chunks of at most 16 tokens, K split over the four waves of a
+// workgroup (16 rows a workgroup): the down step of a few tokens whose matrices have too few
+// 64-row blocks to fill the chip.
+template <int FMT>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_split_kernel(const GemmArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[4 * 2 * 16 * GEMM_A_STRIDE];
+    const int c = blockIdx.y;
+    int e = 0, start, count;
+    if (a.chunk_expert) {
+        if (c >= *a.n_chunks) return;
+        e = a.chunk_expert[c];
+        start = a.chunk_start[c];
+        count = a.chunk_count[c];
+    } else {
+        start = c * GEMM_CHUNK;
+        count = a.dense_tokens - start < GEMM_CHUNK ? a.dense_tokens - start : GEMM_CHUNK;
+    }
+    if (count <= 0) return;
+    tile_gemm_chunk<FMT, GEMM_A_PAIR, false, 1, 1, true>(a, e, start, count, blockIdx.x, lds);
+}
+
 // Several dense matrices (y = W x for `tokens` rows of x each) in one launch: blockIdx.x walks
 // the row blocks of all problems, blockIdx.y the token chunks.
 template <int FMT, int AKIND, int NM>
@@ -902,7 +923,21 @@ static void gemm_launch_f(const GemmArgs& a, int a_kind, dim3 grid, hipStream_t 
     }
 }
 
-int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, hipStream_t s) {
+int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s) {
+    // few tokens, plain rows: the K-split kernel where 64-row workgroups would not fill half the chip
+    const bool split = !pair && a_kind == GEMM_A_PAIR && max_count <= 16 && a.k >= 1024 &&
+                       (int64_t)((a.n + 63) / 64) * chunks < stream_grid() / 2;
+    if (split) {
+        const dim3 sgrid((a.n + 15) / 16, chunks), block(GEMM_THREADS);
+        switch (fmt) {
+        case QMOE_FMT_Q8_0: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q8_0>, sgrid, block, 0, s, a); break;
+        case QMOE_FMT_Q6_K: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q6_K>, sgrid, block, 0, s, a); break;
+        case QMOE_FMT_Q5_K: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q5_K>, sgrid, block, 0, s, a); break;
+        case QMOE_FMT_Q4_K: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q4_K>, sgrid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_BF16>, sgrid, block, 0, s, a); break;
+        }
+        return check_launch("token-tile GEMM (K split)");
+    }
     const int rows_per_wg = pair ? 64 : fmt == QMOE_FMT_Q8_0 ? 64 * GEMM_Q8_PLAIN_TILES : 128;
     const dim3 grid((a.n + rows_per_wg - 1) / rows_per_wg, chunks);
 #define QMOE_GEMM_F(F)                                                  \

@@ -49,8 +49,9 @@ struct GemmDenseArgs {
 };
 
 bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const void* a0, int a_kind, int64_t a_stride);
-// grid = (row blocks, chunks); `chunks` is an upper bound when the list lives on the device
-int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, hipStream_t s);
+// grid = (row blocks, chunks); `chunks` is an upper bound when the list lives on the device,
+// `max_count` the most tokens a chunk can hold in this call
+int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s);
 // fills block_start and launches
 int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s);
 

@@ -221,7 +221,7 @@ int swiglu_impl(const void* gate, int gf, const void* up, int uf, int f, int k, 
         g.dense_tokens = tokens;
         g.out0 = h;
         g.out_dt = hdt;
-        return gemm_launch(gf, true, xdt, g, (tokens + GEMM_CHUNK - 1) / GEMM_CHUNK, s);
+        return gemm_launch(gf, true, xdt, g, (tokens + GEMM_CHUNK - 1) / GEMM_CHUNK, tokens, s);
     }
     const bool xf = x_fast(x, xdt, k);
     const bool gfast = xf && rows_fast(gf, gate, row_bytes(gf, k), k);

@@ -447,7 +447,7 @@ static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L,
     uint16_t* h_lo = h_hi + assignments * b.d_ff;
     g.out0 = h_hi;
     g.out1 = h_lo;
-    if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, s))) return rc;
+    if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, a.tokens, s))) return rc;
     GemmArgs d = g;
     d.w = (const uint8_t*)b.down;
     d.w2 = nullptr;
@@ -461,7 +461,7 @@ static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L,
     d.out0 = ws + L.terms;
     d.out1 = nullptr;
     d.scale = (const float*)(ws + L.sorted_weight);
-    if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, s))) return rc;
+    if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, a.tokens, s))) return rc;
     const float* shared_out = nullptr;
     if (a.shared_gate_w) {
         const int chunks = (a.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
@@ -477,7 +477,7 @@ static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L,
         uint16_t* s_lo = s_hi + (size_t)a.tokens * a.d_ff_shared;
         sg.out0 = s_hi;
         sg.out1 = s_lo;
-        if ((rc = gemm_launch(a.shared_gate_fmt, true, a.hidden_dtype, sg, chunks, s))) return rc;
+        if ((rc = gemm_launch(a.shared_gate_fmt, true, a.hidden_dtype, sg, chunks, a.tokens, s))) return rc;
         GemmArgs sd{};
         sd.w = (const uint8_t*)a.shared_down_w;
         sd.n = b.d_model;
@@ -487,7 +487,7 @@ static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L,
         sd.a_stride = a.d_ff_shared;
         sd.dense_tokens = a.tokens;
         sd.out0 = ws + L.shared_out;
-        if ((rc = gemm_launch(a.shared_down_fmt, false, GEMM_A_PAIR, sd, chunks, s))) return rc;
+        if ((rc = gemm_launch(a.shared_down_fmt, false, GEMM_A_PAIR, sd, chunks, a.tokens, s))) return rc;
         shared_out = (const float*)(ws + L.shared_out);
     }
     return launch_combine(a, ws, L, shared_out, s);
