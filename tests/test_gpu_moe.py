@@ -339,11 +339,13 @@ def test_moe_token_batches_ragged_shapes(cuda, fmt, dtype):
 
 @pytest.mark.parametrize("fmt", ["Q8_0", "Q5_K"])
 @pytest.mark.parametrize("tokens", [1, 3, 16])
-def test_few_tokens_outside_the_decode_shapes(cuda, fmt, tokens):
-    """Expert widths the decode launches do not cover (768 = 6 x 128 columns; a shared expert in
-    another format than the bank): few tokens then take the token-tile GEMMs, same results."""
-    announce("moe few tokens, other shapes", fmt, tokens)
-    e, d, f, fsh, k = 16, 512, 768, 256, 4
+@pytest.mark.parametrize("f", [768, 1280])
+def test_few_tokens_outside_the_decode_shapes(cuda, fmt, tokens, f):
+    """Expert widths the decode launches do not cover (768 = 6 x 128 and 1280 = 10 x 128 columns; a
+    shared expert in another format than the bank): few tokens then take the token-tile GEMMs
+    (the wider down step with K split over the waves of a workgroup), same results."""
+    announce("moe few tokens, other shapes", fmt, tokens, f)
+    e, d, fsh, k = 16, 512, 256, 4
     gate, up, down, _, gate_vec = make_layer(e, d, f, fsh, (fmt, fmt, fmt), 2100)
     shared = (synthetic.packed_weight("Q8_0", (fsh, d), 2101), synthetic.packed_weight("Q8_0", (fsh, d), 2102),
               synthetic.packed_weight("Q6_K", (d, fsh), 2103))
