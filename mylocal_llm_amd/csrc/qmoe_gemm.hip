@@ -615,7 +615,7 @@ __device__ __forceinline__ void q6_tile_loop(const GemmArgs& a, int e, int start
 template <int FMT, int AKIND, bool PAIR, int NM, int MT, bool SOLO>
 __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int start, int count, int rowblock, uint8_t* lds) {
     static_assert(!PAIR || NM == 2, "a pair is two matrices");
-    static_assert(!SOLO || (MT == 1 && !PAIR), "a wave stages one token tile on its own");
+    static_assert(!SOLO || MT == 1, "a wave stages one token tile on its own");
     using U = Unit64<FMT>;
     constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2, NB = BTerms<FMT>::N;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -628,7 +628,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
     int rows[NM];
     const uint8_t* rp[NM];
     if (PAIR) {
-        rows[0] = rows[NM - 1] = rowblock * 64 + wave * 16 + col;
+        rows[0] = rows[NM - 1] = SOLO ? rowblock * 16 + col : rowblock * 64 + wave * 16 + col;
         const int64_t rr = rows[0] < a.n ? rows[0] : a.n - 1;
         rp[0] = a.w + (int64_t)e * a.stride + rr * rb;
         rp[NM - 1] = a.w2 + (int64_t)e * a.stride2 + rr * rb;
@@ -648,7 +648,7 @@ __device__ __forceinline__ void tile_gemm_chunk(const GemmArgs& a, int e, int st
     // lane (col, g) holds outputs of tokens 16*mt + 4*g + i, row index col of each matrix
     auto emit = [&](int block) {
         int rows[NM];
-        if (PAIR) rows[0] = rows[NM - 1] = block * 64 + wave * 16 + col;
+        if (PAIR) rows[0] = rows[NM - 1] = SOLO ? block * 16 + col : block * 64 + wave * 16 + col;
         else {
 #pragma unroll
             for (int j = 0; j < NM; ++j) rows[j] = SOLO ? block * (16 * NM) + 16 * j + col : block * (64 * NM) + wave * (16 * NM) + 16 * j + col;
@@ -849,12 +849,13 @@ __global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)
     else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, blockIdx.x, lds);
 }
 
-// Plain rows over hi/lo activations, chunks of at most 16 tokens, K split over the four waves of a
-// workgroup (16 rows a workgroup): the down step of a few tokens whose matrices have too few
-// 64-row blocks to fill the chip.
-template <int FMT>
+// Chunks of at most 16 tokens with K split over the four waves of a workgroup (16 rows, or 16
+// gate/up row pairs, a workgroup): the steps of a few tokens whose matrices have too few 64-row
+// blocks to fill the chip.
+template <int FMT, int AKIND, bool PAIR>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_split_kernel(const GemmArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[4 * 2 * 16 * GEMM_A_STRIDE];
+    constexpr int NA = AKIND == GEMM_A_BF16 ? 1 : 2;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[4 * NA * 16 * GEMM_A_STRIDE];
     const int c = blockIdx.y;
     int e = 0, start, count;
     if (a.chunk_expert) {
@@ -867,7 +868,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void tile_gemm_split_kernel(const 
         count = a.dense_tokens - start < GEMM_CHUNK ? a.dense_tokens - start : GEMM_CHUNK;
     }
     if (count <= 0) return;
-    tile_gemm_chunk<FMT, GEMM_A_PAIR, false, 1, 1, true>(a, e, start, count, blockIdx.x, lds);
+    tile_gemm_chunk<FMT, AKIND, PAIR, PAIR ? 2 : 1, 1, true>(a, e, start, count, blockIdx.x, lds);
+}
+
+template <int FMT, bool PAIR>
+static void gemm_split_f(const GemmArgs& a, int a_kind, dim3 grid, hipStream_t s) {
+    const dim3 block(GEMM_THREADS);
+    switch (a_kind) {
+    case GEMM_A_F32: hipLaunchKernelGGL((tile_gemm_split_kernel<FMT, GEMM_A_F32, PAIR>), grid, block, 0, s, a); break;
+    case GEMM_A_F16: hipLaunchKernelGGL((tile_gemm_split_kernel<FMT, GEMM_A_F16, PAIR>), grid, block, 0, s, a); break;
+    case GEMM_A_BF16: hipLaunchKernelGGL((tile_gemm_split_kernel<FMT, GEMM_A_BF16, PAIR>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((tile_gemm_split_kernel<FMT, GEMM_A_PAIR, PAIR>), grid, block, 0, s, a); break;
+    }
 }
 
 // Several dense matrices (y = W x for `tokens` rows of x each) in one launch: blockIdx.x walks
@@ -924,18 +936,21 @@ static void gemm_launch_f(const GemmArgs& a, int a_kind, dim3 grid, hipStream_t 
 }
 
 int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s) {
-    // few tokens, plain rows: the K-split kernel where 64-row workgroups would not fill half the chip
-    const bool split = !pair && a_kind == GEMM_A_PAIR && max_count <= 16 && a.k >= 1024 &&
-                       (int64_t)((a.n + 63) / 64) * chunks < stream_grid() / 2;
+    // few tokens: the K-split kernel where 64-row workgroups would not fill half the chip
+    const bool split = max_count <= 16 && a.k >= 1024 && (int64_t)((a.n + 63) / 64) * chunks < stream_grid() / 2;
     if (split) {
-        const dim3 sgrid((a.n + 15) / 16, chunks), block(GEMM_THREADS);
+        const dim3 sgrid((a.n + 15) / 16, chunks);
+#define QMOE_SPLIT_F(F)                                              \
+    if (pair) gemm_split_f<F, true>(a, a_kind, sgrid, s);            \
+    else gemm_split_f<F, false>(a, a_kind, sgrid, s)
         switch (fmt) {
-        case QMOE_FMT_Q8_0: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q8_0>, sgrid, block, 0, s, a); break;
-        case QMOE_FMT_Q6_K: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q6_K>, sgrid, block, 0, s, a); break;
-        case QMOE_FMT_Q5_K: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q5_K>, sgrid, block, 0, s, a); break;
-        case QMOE_FMT_Q4_K: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_Q4_K>, sgrid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL(tile_gemm_split_kernel<QMOE_FMT_BF16>, sgrid, block, 0, s, a); break;
+        case QMOE_FMT_Q8_0: QMOE_SPLIT_F(QMOE_FMT_Q8_0); break;
+        case QMOE_FMT_Q6_K: QMOE_SPLIT_F(QMOE_FMT_Q6_K); break;
+        case QMOE_FMT_Q5_K: QMOE_SPLIT_F(QMOE_FMT_Q5_K); break;
+        case QMOE_FMT_Q4_K: QMOE_SPLIT_F(QMOE_FMT_Q4_K); break;
+        default: QMOE_SPLIT_F(QMOE_FMT_BF16); break;
         }
+#undef QMOE_SPLIT_F
         return check_launch("token-tile GEMM (K split)");
     }
     const int rows_per_wg = pair ? 64 : fmt == QMOE_FMT_Q8_0 ? 64 * GEMM_Q8_PLAIN_TILES : 128;
