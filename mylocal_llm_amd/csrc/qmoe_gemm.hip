@@ -915,9 +915,12 @@ __global__ __launch_bounds__(GEMM_THREADS, (FMT == QMOE_FMT_Q8_0 && AKIND == GEM
 int stream_grid();
 
 bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const void* a0, int a_kind, int64_t a_stride) {
-    if (!stream_supported(fmt, w, n, k, nullptr, QMOE_DT_F32)) return false;  // unit loads: same format and alignment rules
+    // the streaming kernel's formats and alignment rules (same unit loads), rows of any length
+    if (!(fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q4_K || fmt == QMOE_FMT_BF16)) return false;
+    if (k % 64 || n < 1 || k > (1 << 24)) return false;
+    if ((fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q4_K) && (k % 256)) return false;
     const int align = fmt == QMOE_FMT_Q8_0 ? 4 : fmt == QMOE_FMT_Q6_K ? 2 : 16;
-    if (stride % align) return false;
+    if ((uintptr_t)w % align || row_bytes(fmt, k) % align || stride % align) return false;
     // (the tile loops address a matrix with 32-bit offsets)
     if (fmt != QMOE_FMT_BF16 && (int64_t)n * row_bytes(fmt, k) >= (1ll << 32)) return false;
     const int esize = a_kind == GEMM_A_F32 ? 4 : 2;

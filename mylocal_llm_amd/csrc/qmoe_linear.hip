@@ -140,7 +140,9 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
     }
     // token batches: the token-tile GEMM (it splits K over the waves of a workgroup when the matrix
     // alone would leave most of the chip idle); the general kernel where its rules do not hold
-    const bool tile_ok = tokens >= 2 && gemm_supported(fmt, w, 0, n, k, x, xdt, k);
+    // (one token whose row is too long for the streaming kernel's LDS goes the same way if Q8_0;
+    // the K-quants' single token is faster in the general kernel than in the GEMM's K-split loop)
+    const bool tile_ok = (tokens >= 2 || fmt == QMOE_FMT_Q8_0) && gemm_supported(fmt, w, 0, n, k, x, xdt, k);
     if (tile_ok) {
         GemmDenseArgs d{};
         d.count = 1;
@@ -301,7 +303,8 @@ int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stre
         const qmoe_linear_problem& p = problems[i];
         const bool aligned = (uintptr_t)p.x % dtype_size(p.x_dtype) == 0 && (uintptr_t)p.y % dtype_size(p.y_dtype) == 0;
         const bool streams = aligned && p.tokens == 1 && stream_supported(p.fmt, p.w, p.n, p.k, p.x, p.x_dtype);
-        const bool tiles = aligned && p.tokens >= 2 && gemm_supported(p.fmt, p.w, 0, p.n, p.k, p.x, p.x_dtype, p.k);
+        const bool tiles = aligned && !streams && (p.tokens >= 2 || p.fmt == QMOE_FMT_Q8_0) &&
+                           gemm_supported(p.fmt, p.w, 0, p.n, p.k, p.x, p.x_dtype, p.k);
         int rc;
         if (streams) {
             if ((rc = flush_dense())) return rc;

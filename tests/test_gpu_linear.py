@@ -105,6 +105,20 @@ def test_q8_0_token_batches_ragged_rows(cuda, shape, tokens, dtype):
         assert tol <= REL_L2
 
 
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
+@pytest.mark.parametrize("k", [18432, 32768])
+@pytest.mark.parametrize("tokens", [1, 3, 20])
+def test_rows_longer_than_the_streaming_kernel_takes(cuda, fmt, k, tokens):
+    """Rows of more than 16384 columns (the down projections of 70B-class models): the token-tile
+    GEMM has no row-length limit; one token goes there too (Q8_0) or to the general kernel."""
+    announce("linear long rows", fmt, k, tokens)
+    w = synthetic.packed_weight(fmt, (70, k), 411)
+    x = synthetic.activations((tokens, k), 412)
+    want = R.linear(x, *triple(w))
+    got = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    assert rel_l2(got, want) <= 2e-5 <= REL_L2
+
+
 def test_linear_three_dimensional_input_and_shape_errors(cuda):
     w = upload(synthetic.packed_weight("Q4_K", (7, 512), 1), cuda)
     x = torch.from_numpy(synthetic.activations((2, 3, 512), 2)).to(cuda)
