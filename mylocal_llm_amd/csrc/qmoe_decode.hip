@@ -173,10 +173,11 @@ __device__ __forceinline__ StreamProblem decode_problem(const DecodeRouteArgs& a
     return p;
 }
 
+template <int MAXNV>
 __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs a) {
     __shared__ int64_t sid[32];
     const int t = blockIdx.x, lane = threadIdx.x;
-    route_token<64>(a, t, true, sid, [] {});
+    route_token<MAXNV>(a, t, true, sid, [] {});
     __syncthreads();
     const int per_token = a.k + (a.shared_gate_w && !a.shared_apart ? 1 : 0);
     if (lane == 0 && t == 0) *a.problem_count = a.tokens * per_token;
@@ -307,21 +308,54 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void decode_pairs_fused_kernel(c
                 if (t < tokens && col < a.d) xv[t][i] = load_x4(a.hidden, a.xdt, t * a.d + col);
             }
     };
-    if (wave < tokens) route_token<FUSED_MAX_EXPERTS / 64>(a, wave, blockIdx.x == 0, sid[wave], fetch_x);
-    else fetch_x();
+    constexpr int PD = Prefetch<FMT, true>::DEPTH;
+    const int idle = STREAM_WAVES - tokens;   // waves with no token to route
+    if (idle > 0) {
+        // The routing waves only route.  Every other wave stages the activations of all tokens
+        // (each of them writes every value, the same ones, so none waits for another) and takes
+        // its share of the shared expert's gate/up rows, which need no routing: that work
+        // is over by the time the selection rounds are.
+        if (wave < tokens) {
+            route_token<FUSED_MAX_EXPERTS / 64>(a, wave, blockIdx.x == 0, sid[wave], [] {});
+        } else {
+            const int lane = threadIdx.x & 63;
+            for (int t = 0; t < tokens; ++t) {
+                float4 v[16];
 #pragma unroll
-    for (int t = 0; t < FUSED_MAX_TOKENS; ++t)
+                for (int i = 0; i < 16; ++i) {
+                    const int col = 4 * lane + 256 * i;
+                    if (col < a.d) v[i] = load_x4(a.hidden, a.xdt, t * a.d + col);
+                }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int col = 4 * threadIdx.x + 1024 * i;
-            if (t < tokens && col < a.d) *(float4*)(xs + t * STRIPE + StagedX::at(col)) = xv[t][i];
+                for (int i = 0; i < 16; ++i) {
+                    const int col = 4 * lane + 256 * i;
+                    if (col < a.d) *(float4*)(xs + t * STRIPE + StagedX::at(col)) = v[i];
+                }
+            }
+            if (a.shared_gate_w)
+                stream_rows_many_x<FMT, true, PD>(a.shared_gate_w, a.shared_up_w, a.fsh, a.d, xs, STRIPE, tokens, a.hs, a.fsh,
+                                                  blockIdx.x * idle + (wave - tokens), gridDim.x * idle);
         }
-    __syncthreads();
-    const int per_token = k + (a.shared_gate_w ? 1 : 0);
-    const int count = tokens * per_token;
+        __syncthreads();
+    } else {
+        route_token<FUSED_MAX_EXPERTS / 64>(a, wave, blockIdx.x == 0, sid[wave], fetch_x);
+#pragma unroll
+        for (int t = 0; t < FUSED_MAX_TOKENS; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = 4 * threadIdx.x + 1024 * i;
+                if (t < tokens && col < a.d) *(float4*)(xs + t * STRIPE + StagedX::at(col)) = xv[t][i];
+            }
+        __syncthreads();
+        // the shared expert's rows once for all tokens
+        if (a.shared_gate_w)
+            stream_rows_many_x<FMT, true, PD>(a.shared_gate_w, a.shared_up_w, a.fsh, a.d, xs, STRIPE, tokens, a.hs, a.fsh,
+                                              blockIdx.x * STREAM_WAVES + wave, gridDim.x * STREAM_WAVES);
+    }
+    const int count = tokens * k;
     if ((int)threadIdx.x < count) {
-        const int t = threadIdx.x / per_token, j = threadIdx.x % per_token;
-        staged[threadIdx.x] = decode_problem(a, t, j, j < k ? sid[t][j] : 0);
+        const int t = threadIdx.x / k, j = threadIdx.x % k;
+        staged[threadIdx.x] = decode_problem(a, t, j, sid[t][j]);
     }
     __syncthreads();
     stream_run<FMT, true, false>(staged, count, 0, staged[count - 1].flat_end, tokens > 1, nullptr, xs, xs);
@@ -519,10 +553,10 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     r.tokens = a.tokens;
     r.workers = grid * STREAM_WAVES;
     int rc;
-    r.shared_apart = 0;
     const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.top_k + 1 <= FUSED_MAX_SLOTS && b.d_model <= 4096 &&
                        (!a.logits || b.n_experts <= FUSED_MAX_EXPERTS);
     if (fused) {
+        r.shared_apart = has_shared;   // streamed once for all tokens, beside the routing
         const dim3 fg(grid), fb(STREAM_THREADS);
         switch (b.gate_fmt) {
         case QMOE_FMT_Q8_0: hipLaunchKernelGGL(decode_pairs_fused_kernel<QMOE_FMT_Q8_0>, fg, fb, 0, s, r); break;
@@ -534,7 +568,10 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
         if ((rc = check_launch("qmoe_moe_forward(route + gate/up)"))) return rc;
     } else {
     r.shared_apart = has_shared && b.d_model <= 4096 && a.tokens >= 2;
-    hipLaunchKernelGGL(decode_route_kernel, dim3(a.tokens), dim3(64), 0, s, r);
+    // the narrow instance is a fraction of the code: a kernel that runs once per step fetches
+    // its instructions cold
+    if (!a.logits || b.n_experts <= 1024) hipLaunchKernelGGL(decode_route_kernel<16>, dim3(a.tokens), dim3(64), 0, s, r);
+    else hipLaunchKernelGGL(decode_route_kernel<64>, dim3(a.tokens), dim3(64), 0, s, r);
     if ((rc = check_launch("qmoe_moe_forward(route)"))) return rc;
 #define QMOE_LIST(F) hipLaunchKernelGGL((stream_list_kernel<F, true>), dim3(grid), dim3(STREAM_THREADS), 0, s, \
                                         (const StreamProblem*)w.problems, (const int*)w.problem_count, r)
