@@ -47,6 +47,7 @@ struct DecodeRouteArgs {
     int renorm, n_experts, k, d, f, fsh, fmt, xdt, tokens, workers;
     int shared_apart;          // the shared expert's gate/up is not in the problem list: its rows are
                                // streamed once for all tokens by a phase of its own
+    int shared_in_front;       // ... and that phase runs beside the routing, in the routing launch
 };
 
 // hidden[t] . g for the shared expert's admission gate, 2048 columns at a time: issue() only
@@ -184,37 +185,75 @@ __global__ __launch_bounds__(64) void decode_route_kernel(const DecodeRouteArgs 
     if (lane < per_token) a.problems[(size_t)t * per_token + lane] = decode_problem(a, t, lane, lane < a.k ? sid[lane] : 0);
 }
 
-// The shared expert's gate/up rows for all tokens of the step: tokens are staged in LDS in groups
-// (as many padded rows as fit), every workgroup stages the same group, and the rows are streamed
-// once per group instead of once per token.  Workgroup-uniform; ends with the LDS free again.
+// Activation rows of tokens t0 .. t0 + nt - 1 into padded LDS stripes, by the whole workgroup.
+// A token's loads are issued together, then stored (a store between two loads orders them).
+// (All tokens' loads ahead of all stores measured slower.)
+__device__ __forceinline__ void stage_tokens(const DecodeRouteArgs& a, float* xs, int stripe, int t0, int nt) {
+    for (int i = 0; i < nt; ++i) {
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+            if (c < a.d) v[j] = load_x4(a.hidden, a.xdt, (t0 + i) * a.d + c);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
+            if (c < a.d) *(float4*)(xs + i * stripe + StagedX::at(c)) = v[j];
+        }
+    }
+}
+
+// The shared expert's gate/up rows for all tokens of the step.  The tokens are cut into groups
+// whose activations fit the LDS stripes together; workgroup `wg` of `wgs` serves group
+// wg % groups: it stages that group's tokens and shares the rows with the other workgroups of
+// the group, every row streamed once per group and reduced against each staged token in turn.
+// A wave's chain (row fetch, then one reduction per token of its group) is pure latency, so
+// the tokens are cut into more groups than LDS asks for as long as that gives waves a row that
+// would have none.  Workgroup-uniform; ends with the LDS free again.
 template <int FMT>
-__device__ __forceinline__ void shared_pairs_phase(const DecodeRouteArgs& a, float* xs) {
+__device__ __forceinline__ void shared_pairs_phase(const DecodeRouteArgs& a, float* xs, int wg, int wgs) {
     const int stripe = a.d + 4 * (a.d >> 6);
     const int fit = STREAM_XS_FLOATS / stripe;
     const int wave = threadIdx.x >> 6;
-    for (int t0 = 0; t0 < a.tokens; t0 += fit) {
-        const int groups = a.tokens - t0 < fit ? a.tokens - t0 : fit;
+    const int rpw = 64 / lanes_per_row(a.d);
+    const long items = (a.fsh + rpw - 1) / rpw;
+    int groups = (a.tokens + fit - 1) / fit;
+    while (2 * groups <= a.tokens && 2 * groups <= wgs && items * 2 * groups <= (long)wgs * STREAM_WAVES * 21 / 20) groups *= 2;
+    const int per = (a.tokens + groups - 1) / groups;
+    for (int g = wg % groups; g < groups; g += wgs) {
+        const int t0 = g * per;
+        const int nt = a.tokens - t0 < per ? a.tokens - t0 : per;
+        if (nt <= 0) break;
+        const int serving = wgs >= groups ? (wgs - g + groups - 1) / groups : 1;   // workgroups of this group
+        const int mine = wgs >= groups ? wg / groups : 0;
         __syncthreads();
-        // a token's loads are issued together, then stored (a store between two loads orders them)
-        for (int g = 0; g < groups; ++g) {
-            float4 v[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
-                if (i < a.d) v[j] = load_x4(a.hidden, a.xdt, (t0 + g) * a.d + i);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
-                if (i < a.d) *(float4*)(xs + g * stripe + StagedX::at(i)) = v[j];
-            }
-        }
+        stage_tokens(a, xs, stripe, t0, nt);
         __syncthreads();
-        stream_rows_many_x<FMT, true, Prefetch<FMT, true>::DEPTH>(a.shared_gate_w, a.shared_up_w, a.fsh, a.d, xs, stripe, groups,
+        stream_rows_many_x<FMT, true, Prefetch<FMT, true>::DEPTH>(a.shared_gate_w, a.shared_up_w, a.fsh, a.d, xs, stripe, nt,
                                                                  a.hs + (size_t)t0 * a.fsh, a.fsh,
-                                                                 blockIdx.x * STREAM_WAVES + wave, gridDim.x * STREAM_WAVES);
+                                                                 mine * STREAM_WAVES + wave, serving * STREAM_WAVES);
     }
     __syncthreads();
+}
+
+// Routing and the shared expert's gate/up rows in one launch (the rows need no routing):
+// workgroup t < tokens routes token t with its first wave, as decode_route_kernel does; all
+// other workgroups stream.  The launch is as long as the longer of the two.
+template <int FMT>
+__global__ __launch_bounds__(STREAM_THREADS, 2) void decode_front_kernel(const DecodeRouteArgs a) {
+    __shared__ int64_t sid[32];
+    __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
+    if ((int)blockIdx.x < a.tokens) {
+        if (threadIdx.x >= 64) return;
+        const int t = blockIdx.x, lane = threadIdx.x;
+        route_token<16>(a, t, true, sid, [] {});
+        __builtin_amdgcn_wave_barrier();   // one wave: its LDS accesses complete in order
+        if (lane == 0 && t == 0) *a.problem_count = a.tokens * a.k;
+        if (lane < a.k) a.problems[(size_t)t * a.k + lane] = decode_problem(a, t, lane, sid[lane]);
+        return;
+    }
+    shared_pairs_phase<FMT>(a, xs, blockIdx.x - a.tokens, gridDim.x - a.tokens);
 }
 
 // The streaming engine over a problem list that lives in device memory.
@@ -225,7 +264,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
     __shared__ float partial[32 * 2 * 4];
     __shared__ StreamProblem staged[LIST_STAGE];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
-    if (a.shared_apart) shared_pairs_phase<FMT>(a, xs);
+    if (a.shared_apart && !a.shared_in_front) shared_pairs_phase<FMT>(a, xs, blockIdx.x, gridDim.x);
     const int n = *count;
     const int units = a.d >> 6;
     if (units <= 64) {
@@ -247,19 +286,7 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_list_kernel(const St
             const uint4* src = (const uint4*)(list + base);
             uint4* dst = (uint4*)staged;
             for (int i = threadIdx.x; i < m * 4; i += STREAM_THREADS) dst[i] = src[i];
-            for (int g = 0; g < nt; ++g) {
-                float4 v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
-                    if (i < a.d) v[j] = load_x4(a.hidden, a.xdt, (t0 + g) * a.d + i);
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int i = 4 * threadIdx.x + 4 * STREAM_THREADS * j;
-                    if (i < a.d) *(float4*)(xs + g * stripe + StagedX::at(i)) = v[j];
-                }
-            }
+            stage_tokens(a, xs, stripe, t0, nt);
             __syncthreads();
             if ((int)threadIdx.x < m) staged[threadIdx.x].xgroup -= t0;   // stripe of the token inside this group
             __syncthreads();
@@ -568,6 +595,17 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
         if ((rc = check_launch("qmoe_moe_forward(route + gate/up)"))) return rc;
     } else {
     r.shared_apart = has_shared && b.d_model <= 4096 && a.tokens >= 2;
+    r.shared_in_front = r.shared_apart && (!a.logits || b.n_experts <= 1024) && grid > 2 * a.tokens;
+    if (r.shared_in_front) {
+        const dim3 fg(grid), fb(STREAM_THREADS);
+        switch (b.gate_fmt) {
+        case QMOE_FMT_Q8_0: hipLaunchKernelGGL(decode_front_kernel<QMOE_FMT_Q8_0>, fg, fb, 0, s, r); break;
+        case QMOE_FMT_Q6_K: hipLaunchKernelGGL(decode_front_kernel<QMOE_FMT_Q6_K>, fg, fb, 0, s, r); break;
+        case QMOE_FMT_Q5_K: hipLaunchKernelGGL(decode_front_kernel<QMOE_FMT_Q5_K>, fg, fb, 0, s, r); break;
+        case QMOE_FMT_Q4_K: hipLaunchKernelGGL(decode_front_kernel<QMOE_FMT_Q4_K>, fg, fb, 0, s, r); break;
+        default: hipLaunchKernelGGL(decode_front_kernel<QMOE_FMT_BF16>, fg, fb, 0, s, r); break;
+        }
+    } else
     // the narrow instance is a fraction of the code: a kernel that runs once per step fetches
     // its instructions cold
     if (!a.logits || b.n_experts <= 1024) hipLaunchKernelGGL(decode_route_kernel<16>, dim3(a.tokens), dim3(64), 0, s, r);
