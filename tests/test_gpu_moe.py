@@ -395,6 +395,7 @@ def test_decode_path_with_more_experts_than_the_fused_launch_routes(cuda, tokens
     (8, 2048, 512, 0, 4, "Q6_K", 5, "f32"),       # no shared expert
     (8, 1024, 256, 512, 3, "Q4_K", 2, "f32"),     # Q4_K bank: fused kernel
     (8, 1024, 256, 512, 3, "Q4_K", 7, "bf16"),    # Q4_K bank: routing kernel + list
+    (8, 4096, 128, 256, 2, "Q8_0", 11, "bf16"),   # 4096 columns: four tokens fit the LDS stripes, uneven token groups
 ])
 def test_decode_shapes_lane_layouts_and_types(cuda, e, d, f, fsh, k, fmt, tokens, dtype):
     """Decode-size steps across the lane layouts of the two kernels (row widths of the gate/up
