@@ -18,11 +18,13 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamA
     __shared__ StreamProblem probs[STREAM_MAX_PROBLEMS];
     __shared__ __attribute__((aligned(16))) float xs[STREAM_XS_FLOATS];
     if ((int)threadIdx.x < args.count) probs[threadIdx.x] = args.p[threadIdx.x];
-    // every activation row the flat stream will need, fetched together: a wave that moves on to
-    // the next matrix finds its activations in LDS instead of waiting for them
+    // Every activation row the flat stream will need is fetched at the start: a wave that moves
+    // on to the next matrix finds its activations in LDS instead of waiting for them.  The
+    // loads leave first; the wave then requests its first weight rows, and only then stores the
+    // activations (which arrive first) and meets the other waves: the rows travel meanwhile.
+    constexpr int STRIPE = STREAM_XS_FLOATS / STREAM_WAVES;
+    float4 v[STREAM_WAVES][4];
     if (args.groups > 0) {
-        constexpr int STRIPE = STREAM_XS_FLOATS / STREAM_WAVES;
-        float4 v[STREAM_WAVES][4];
 #pragma unroll
         for (int g = 0; g < STREAM_WAVES; ++g) {
             const StreamProblem& p = args.p[args.group_problem[g < args.groups ? g : 0]];
@@ -32,18 +34,30 @@ __global__ __launch_bounds__(STREAM_THREADS, 2) void stream_kernel(const StreamA
                 if (g < args.groups && col < p.k) v[g][i] = load_x4(p.x, p.xdt, col);
             }
         }
+    }
+    __syncthreads();   // the problem list is in LDS
+    auto store_x = [&] {
+        if (args.groups > 0) {
 #pragma unroll
-        for (int g = 0; g < STREAM_WAVES; ++g) {
-            const int pk = args.p[args.group_problem[g < args.groups ? g : 0]].k;
+            for (int g = 0; g < STREAM_WAVES; ++g) {
+                const int pk = args.p[args.group_problem[g < args.groups ? g : 0]].k;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int col = 4 * threadIdx.x + 1024 * i;
-                if (g < args.groups && col < pk) *(float4*)(xs + g * STRIPE + StagedX::at(col)) = v[g][i];
+                for (int i = 0; i < 4; ++i) {
+                    const int col = 4 * threadIdx.x + 1024 * i;
+                    if (g < args.groups && col < pk) *(float4*)(xs + g * STRIPE + StagedX::at(col)) = v[g][i];
+                }
             }
         }
+        __syncthreads();
+    };
+    // (measured per format: Q6_K, whose rows are requested two steps ahead, is faster the plain way)
+    if (FMT == QMOE_FMT_Q6_K) {
+        store_x();
+        stream_run<FMT, PAIR, true>(probs, args.count, 0, args.flat_items, false, partial, xs, args.groups > 0 ? xs : nullptr);
+    } else {
+        stream_run<FMT, PAIR, true>(probs, args.count, 0, args.flat_items, false, partial, xs, args.groups > 0 ? xs : nullptr,
+                                    STREAM_XS_FLOATS / STREAM_WAVES, store_x);
     }
-    __syncthreads();
-    stream_run<FMT, PAIR>(probs, args.count, 0, args.flat_items, false, partial, xs, args.groups > 0 ? xs : nullptr);
 }
 
 // ---- host side ---------------------------------------------------------------------------------

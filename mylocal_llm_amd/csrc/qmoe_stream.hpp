@@ -564,9 +564,14 @@ __device__ __forceinline__ const uint8_t* uniform(const uint8_t* p) {
 // the lane's 64-value slice; with `xpre` the caller has already put the activations of
 // xgroup g into stripe g of that array (same padded layout, stripes `xstride` floats apart) and
 // nothing is fetched here.  Items [begin, end) are walked; `probs` covers them in order.
-template <int FMT, bool PAIR, int PD>
+// `between` runs once on every wave, after the wave's first PD row requests have left and before
+// anything is read from the stripes: a caller whose activations are still on their way stores
+// them (and meets the workgroup's other waves) there, while the rows travel.
+struct NothingBetween { __device__ __forceinline__ void operator()() const {} };
+template <int FMT, bool PAIR, int PD, class Between = NothingBetween>
 __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int count, int begin, int end, bool contiguous, float* xw,
-                                            const float* xpre, int xstride = STREAM_XS_FLOATS / STREAM_WAVES) {
+                                            const float* xpre, int xstride = STREAM_XS_FLOATS / STREAM_WAVES,
+                                            Between&& between = Between()) {
     using U = Unit64<FMT>;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int W = gridDim.x * STREAM_WAVES;
@@ -578,7 +583,10 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
         end = g + share + (me < extra ? 1 : 0);
         step = 1;
     }
-    if (g >= end) return;
+    if (g >= end) {
+        between();
+        return;
+    }
     RowRegs<FMT, PAIR> buf[PD + 1];
     int bp[PD + 1], bi[PD + 1];
     // the problem the fetch side is in, held in scalar registers
@@ -622,6 +630,7 @@ __device__ __forceinline__ void stream_flat(const StreamProblem* probs, int coun
     auto bounded = [&](int gi) { return gi < end ? gi : last; };
 #pragma unroll
     for (int j = 0; j < PD; ++j) fetch(bounded(g + j * step), g + j * step >= end, buf[j], bp[j], bi[j]);
+    between();
     float xr[64], aux[8];
     int xgroup = -1;
     bool done = false;
@@ -737,13 +746,16 @@ template <int FMT, bool PAIR> struct Prefetch {
 
 // A whole problem list held in LDS: first the single stream of all problems whose rows fit a
 // wave, then, one after the other, the problems with wider rows (four waves per row).
-template <int FMT, bool PAIR, bool WIDE = true>
+template <int FMT, bool PAIR, bool WIDE = true, class Between = NothingBetween>
 __device__ __forceinline__ void stream_run(const StreamProblem* probs, int count, int flat_begin, int flat_end, bool contiguous, float* partial, float* xs,
-                                           const float* xpre = nullptr, int xstride = STREAM_XS_FLOATS / STREAM_WAVES) {
+                                           const float* xpre = nullptr, int xstride = STREAM_XS_FLOATS / STREAM_WAVES,
+                                           Between&& between = Between()) {
     constexpr int PD = Prefetch<FMT, PAIR>::DEPTH;
     const int wave = threadIdx.x >> 6;
     if (flat_end > flat_begin)
-        stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES), xpre, xstride);
+        stream_flat<FMT, PAIR, PD>(probs, count, flat_begin, flat_end, contiguous, xs + wave * (STREAM_XS_FLOATS / STREAM_WAVES), xpre, xstride, between);
+    else
+        between();
     if (!WIDE) return;
     float xr[64], aux[8];
     int xgroup = -1, staged = -1;
