@@ -235,7 +235,26 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     }
     if (shared_out && shared_gate) {
         float a = 0.0f;
-        for (int i = tid; i < d; i += 256) a += Elem<XDT>::load(x, (size_t)t * d + i) * shared_gate[i];
+        if ((d & 3) == 0 && (((size_t)shared_gate | (size_t)x) & 15) == 0) {
+            // up to four pieces a thread, loads first
+            float4 h[4], g[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = 4 * tid + 1024 * j;
+                const bool in = i < d;
+                h[j] = Elem<XDT>::load4(x, (size_t)t * d + (in ? i : 0));
+                g[j] = ldg<float4>(shared_gate + (in ? i : 0));
+                if (!in) g[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) a += (h[j].x * g[j].x + h[j].y * g[j].y) + (h[j].z * g[j].z + h[j].w * g[j].w);
+            for (int i = 4 * tid + 4096; i < d; i += 1024) {
+                const float4 hh = Elem<XDT>::load4(x, (size_t)t * d + i), gg = ldg<float4>(shared_gate + i);
+                a += (hh.x * gg.x + hh.y * gg.y) + (hh.z * gg.z + hh.w * gg.w);
+            }
+        } else {
+            for (int i = tid; i < d; i += 256) a += Elem<XDT>::load(x, (size_t)t * d + i) * shared_gate[i];
+        }
         a = wave_sum(a);
         if ((tid & 63) == 0) partial[tid >> 6] = a;
         __syncthreads();
@@ -252,12 +271,23 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
         // each column stay in ascending expert order
         for (int i = 4 * tid; i < d; i += 4 * 256) {
             float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int s = 0; s < k; ++s) {
-                const int p = order[s];
-                if (p >= 0) {
-                    const float4 v = *(const float4*)(terms + (size_t)p * d + i);
-                    acc.x = __fadd_rn(acc.x, v.x); acc.y = __fadd_rn(acc.y, v.y);
-                    acc.z = __fadd_rn(acc.z, v.z); acc.w = __fadd_rn(acc.w, v.w);
+            // eight terms at a time: their loads leave together (an absent one reads row 0 and is
+            // not added), the adds follow in order
+            for (int s0 = 0; s0 < k; s0 += 8) {
+                float4 v[8];
+                bool live[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int p = s0 + j < k ? order[s0 + j] : -1;
+                    live[j] = p >= 0;
+                    v[j] = ldg<float4>(terms + (size_t)(live[j] ? p : 0) * d + i);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (live[j]) {
+                        acc.x = __fadd_rn(acc.x, v[j].x); acc.y = __fadd_rn(acc.y, v[j].y);
+                        acc.z = __fadd_rn(acc.z, v[j].z); acc.w = __fadd_rn(acc.w, v[j].w);
+                    }
                 }
             }
             if (shared_out) {
