@@ -829,11 +829,26 @@ template <int FMT, int AKIND, bool PAIR> struct GroupedShape {
     static constexpr int WGS = (WeightTile<FMT, NM>::BYTES != 0 && LDS * 3 <= 160 * 1024) ? GEMM_SLIM_WGS : 2;
 };
 
+// A launch may carry a second, dense problem of the same kinds (`side`: the shared expert beside
+// the routed ones): its token chunks come first in blockIdx.y, each cut into `side_parts` parts
+// of gridDim.x row blocks, so that the two problems need not have the same number of rows and
+// the long workgroups of the dense problem start first.
 template <int FMT, int AKIND, bool PAIR>
-__global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)) void tile_gemm_kernel(const GemmArgs a) {
+__global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)) void tile_gemm_kernel(const GemmArgs main_args, const GemmArgs side,
+                                                                                                       int side_chunks, int side_parts) {
     using GS = GroupedShape<FMT, AKIND, PAIR>;
     __shared__ __attribute__((aligned(16))) uint8_t lds[GS::LDS];
-    const int c = blockIdx.y;
+    constexpr int ROWS_PER_WG = PAIR ? 64 : 64 * GS::NM;
+    int c = blockIdx.y, rowblock = blockIdx.x;
+    const bool on_side = c < side_chunks * side_parts;
+    const GemmArgs& a = on_side ? side : main_args;
+    if (on_side) {
+        rowblock += (c % side_parts) * gridDim.x;
+        c /= side_parts;
+    } else {
+        c -= side_chunks * side_parts;
+    }
+    if (rowblock * ROWS_PER_WG >= a.n) return;
     int e = 0, start, count;
     if (a.chunk_expert) {
         if (c >= *a.n_chunks) return;
@@ -845,8 +860,8 @@ __global__ __launch_bounds__(GEMM_THREADS, (GroupedShape<FMT, AKIND, PAIR>::WGS)
         count = a.dense_tokens - start < GEMM_CHUNK ? a.dense_tokens - start : GEMM_CHUNK;
     }
     if (count <= 0) return;
-    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 1, false>(a, e, start, count, blockIdx.x, lds);
-    else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, blockIdx.x, lds);
+    if (count <= 16) tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 1, false>(a, e, start, count, rowblock, lds);
+    else tile_gemm_chunk<FMT, AKIND, PAIR, GS::NM, 2, false>(a, e, start, count, rowblock, lds);
 }
 
 // Chunks of at most 16 tokens with K split over the four waves of a workgroup (16 rows, or 16
@@ -928,19 +943,28 @@ bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const 
 }
 
 template <int FMT, bool PAIR>
-static void gemm_launch_f(const GemmArgs& a, int a_kind, dim3 grid, hipStream_t s) {
+static void gemm_launch_f(const GemmArgs& a, const GemmArgs& side, int side_chunks, int side_parts, int a_kind, dim3 grid, hipStream_t s) {
     const dim3 block(GEMM_THREADS);
     switch (a_kind) {
-    case GEMM_A_F32: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_F32, PAIR>), grid, block, 0, s, a); break;
-    case GEMM_A_F16: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_F16, PAIR>), grid, block, 0, s, a); break;
-    case GEMM_A_BF16: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_BF16, PAIR>), grid, block, 0, s, a); break;
-    default: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_PAIR, PAIR>), grid, block, 0, s, a); break;
+    case GEMM_A_F32: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_F32, PAIR>), grid, block, 0, s, a, side, side_chunks, side_parts); break;
+    case GEMM_A_F16: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_F16, PAIR>), grid, block, 0, s, a, side, side_chunks, side_parts); break;
+    case GEMM_A_BF16: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_BF16, PAIR>), grid, block, 0, s, a, side, side_chunks, side_parts); break;
+    default: hipLaunchKernelGGL((tile_gemm_kernel<FMT, GEMM_A_PAIR, PAIR>), grid, block, 0, s, a, side, side_chunks, side_parts); break;
     }
 }
 
-int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s) {
+static bool gemm_splits_k(const GemmArgs& a, int chunks, int max_count) {
+    return max_count <= 16 && a.k >= 1024 && (int64_t)((a.n + 63) / 64) * chunks < stream_grid() / 2;
+}
+
+bool gemm_side_fits(const GemmArgs& a, int chunks, const GemmArgs& side, int side_chunks, int max_count) {
+    return !gemm_splits_k(a, chunks, max_count) && !gemm_splits_k(side, side_chunks, max_count) && !side.chunk_expert && side.n >= 1;
+}
+
+int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s,
+                const GemmArgs* side, int side_chunks) {
     // few tokens: the K-split kernel where 64-row workgroups would not fill half the chip
-    const bool split = max_count <= 16 && a.k >= 1024 && (int64_t)((a.n + 63) / 64) * chunks < stream_grid() / 2;
+    const bool split = !side && gemm_splits_k(a, chunks, max_count);
     if (split) {
         const dim3 sgrid((a.n + 15) / 16, chunks);
 #define QMOE_SPLIT_F(F)                                              \
@@ -957,10 +981,16 @@ int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, i
         return check_launch("token-tile GEMM (K split)");
     }
     const int rows_per_wg = pair ? 64 : fmt == QMOE_FMT_Q8_0 ? 64 * GEMM_Q8_PLAIN_TILES : 128;
-    const dim3 grid((a.n + rows_per_wg - 1) / rows_per_wg, chunks);
-#define QMOE_GEMM_F(F)                                                  \
-    if (pair) gemm_launch_f<F, true>(a, a_kind, grid, s);               \
-    else gemm_launch_f<F, false>(a, a_kind, grid, s)
+    const int rowblocks = (a.n + rows_per_wg - 1) / rows_per_wg;
+    // the side problem's row blocks in parts of the main problem's grid width
+    const int side_parts = side ? ((side->n + rows_per_wg - 1) / rows_per_wg + rowblocks - 1) / rowblocks : 0;
+    const GemmArgs none{};
+    const GemmArgs& sd = side ? *side : none;
+    const int sc = side ? side_chunks : 0;
+    const dim3 grid(rowblocks, chunks + sc * side_parts);
+#define QMOE_GEMM_F(F)                                                          \
+    if (pair) gemm_launch_f<F, true>(a, sd, sc, side_parts, a_kind, grid, s);   \
+    else gemm_launch_f<F, false>(a, sd, sc, side_parts, a_kind, grid, s)
     switch (fmt) {
     case QMOE_FMT_Q8_0: QMOE_GEMM_F(QMOE_FMT_Q8_0); break;
     case QMOE_FMT_Q6_K: QMOE_GEMM_F(QMOE_FMT_Q6_K); break;

@@ -51,7 +51,11 @@ struct GemmDenseArgs {
 bool gemm_supported(int fmt, const void* w, int64_t stride, int n, int k, const void* a0, int a_kind, int64_t a_stride);
 // grid = (row blocks, chunks); `chunks` is an upper bound when the list lives on the device,
 // `max_count` the most tokens a chunk can hold in this call
-int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s);
+// `side`: a dense problem (null chunk_expert, `side_chunks` chunks of its dense_tokens) of the same
+// format, pairing and activation kind that shares the launch; only where gemm_side_fits says so
+int gemm_launch(int fmt, bool pair, int a_kind, const GemmArgs& a, int chunks, int max_count, hipStream_t s,
+                const GemmArgs* side = nullptr, int side_chunks = 0);
+bool gemm_side_fits(const GemmArgs& a, int chunks, const GemmArgs& side, int side_chunks, int max_count);
 // fills block_start and launches
 int gemm_dense_launch(int fmt, int a_kind, GemmDenseArgs& d, hipStream_t s);
 

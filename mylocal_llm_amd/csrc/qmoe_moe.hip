@@ -477,7 +477,6 @@ static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L,
     uint16_t* h_lo = h_hi + assignments * b.d_ff;
     g.out0 = h_hi;
     g.out1 = h_lo;
-    if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, a.tokens, s))) return rc;
     GemmArgs d = g;
     d.w = (const uint8_t*)b.down;
     d.w2 = nullptr;
@@ -491,35 +490,49 @@ static int gemm_forward(const qmoe_moe_args& a, char* ws, const MoeWorkspace& L,
     d.out0 = ws + L.terms;
     d.out1 = nullptr;
     d.scale = (const float*)(ws + L.sorted_weight);
-    if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, a.tokens, s))) return rc;
     const float* shared_out = nullptr;
-    if (a.shared_gate_w) {
-        const int chunks = (a.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
-        GemmArgs sg{};
-        sg.w = (const uint8_t*)a.shared_gate_w;
-        sg.w2 = (const uint8_t*)a.shared_up_w;
-        sg.n = a.d_ff_shared;
-        sg.k = b.d_model;
-        sg.a0 = a.hidden;
-        sg.a_stride = b.d_model;
-        sg.dense_tokens = a.tokens;
-        uint16_t* s_hi = (uint16_t*)(ws + L.shared_h);
-        uint16_t* s_lo = s_hi + (size_t)a.tokens * a.d_ff_shared;
-        sg.out0 = s_hi;
-        sg.out1 = s_lo;
-        if ((rc = gemm_launch(a.shared_gate_fmt, true, a.hidden_dtype, sg, chunks, a.tokens, s))) return rc;
-        GemmArgs sd{};
-        sd.w = (const uint8_t*)a.shared_down_w;
-        sd.n = b.d_model;
-        sd.k = a.d_ff_shared;
-        sd.a0 = s_hi;
-        sd.a1 = s_lo;
-        sd.a_stride = a.d_ff_shared;
-        sd.dense_tokens = a.tokens;
-        sd.out0 = ws + L.shared_out;
-        if ((rc = gemm_launch(a.shared_down_fmt, false, GEMM_A_PAIR, sd, chunks, a.tokens, s))) return rc;
-        shared_out = (const float*)(ws + L.shared_out);
+    if (!a.shared_gate_w) {
+        if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, a.tokens, s))) return rc;
+        if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, a.tokens, s))) return rc;
+        return launch_combine(a, ws, L, shared_out, s);
     }
+    const int chunks = (a.tokens + GEMM_CHUNK - 1) / GEMM_CHUNK;
+    GemmArgs sg{};
+    sg.w = (const uint8_t*)a.shared_gate_w;
+    sg.w2 = (const uint8_t*)a.shared_up_w;
+    sg.n = a.d_ff_shared;
+    sg.k = b.d_model;
+    sg.a0 = a.hidden;
+    sg.a_stride = b.d_model;
+    sg.dense_tokens = a.tokens;
+    uint16_t* s_hi = (uint16_t*)(ws + L.shared_h);
+    uint16_t* s_lo = s_hi + (size_t)a.tokens * a.d_ff_shared;
+    sg.out0 = s_hi;
+    sg.out1 = s_lo;
+    GemmArgs sd{};
+    sd.w = (const uint8_t*)a.shared_down_w;
+    sd.n = b.d_model;
+    sd.k = a.d_ff_shared;
+    sd.a0 = s_hi;
+    sd.a1 = s_lo;
+    sd.a_stride = a.d_ff_shared;
+    sd.dense_tokens = a.tokens;
+    sd.out0 = ws + L.shared_out;
+    // The shared expert's two GEMMs ride in the routed launches (its gate/up needs no routing, its
+    // down needs only its own gate/up): on their own they are short launches of few, long
+    // workgroups that leave most of the chip waiting.
+    const bool together = a.shared_gate_fmt == b.gate_fmt && a.shared_down_fmt == b.down_fmt &&
+                          gemm_side_fits(g, L.max_chunks, sg, chunks, a.tokens) && gemm_side_fits(d, L.max_chunks, sd, chunks, a.tokens);
+    if (together) {
+        if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, a.tokens, s, &sg, chunks))) return rc;
+        if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, a.tokens, s, &sd, chunks))) return rc;
+    } else {
+        if ((rc = gemm_launch(b.gate_fmt, true, a.hidden_dtype, g, L.max_chunks, a.tokens, s))) return rc;
+        if ((rc = gemm_launch(b.down_fmt, false, GEMM_A_PAIR, d, L.max_chunks, a.tokens, s))) return rc;
+        if ((rc = gemm_launch(a.shared_gate_fmt, true, a.hidden_dtype, sg, chunks, a.tokens, s))) return rc;
+        if ((rc = gemm_launch(a.shared_down_fmt, false, GEMM_A_PAIR, sd, chunks, a.tokens, s))) return rc;
+    }
+    shared_out = (const float*)(ws + L.shared_out);
     return launch_combine(a, ws, L, shared_out, s);
 }
 
