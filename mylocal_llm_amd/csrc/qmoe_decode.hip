@@ -429,7 +429,8 @@ __global__ __launch_bounds__(256, 2) void decode_down_kernel(const DecodeDownArg
     const bool shared = lane >= 48 && lane - 48 < shared_parts;
     const int slot = routed ? lane / LPE : 0;
     const int part = routed ? lane % LPE : (shared ? lane - 48 : 0);
-    const int e = routed ? a.sorted_ids[(size_t)t * k + slot] : 0;
+    // lanes with nothing to do read what lane 0 reads (its expert, part 0): no cache line of their own
+    const int e = a.sorted_ids[(size_t)t * k + slot];
     const float route_w = lane < k ? a.sorted_w[(size_t)t * k + lane] : 0.f;  // lane j holds weight j
     const bool live = (routed && e >= 0) || shared;
     const int kk = shared ? a.fsh : a.f;
