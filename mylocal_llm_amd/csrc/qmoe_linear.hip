@@ -7,6 +7,7 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include "qmoe_few.hpp"
 #include "qmoe_gemm.hpp"
 #include "qmoe_rowdot.hpp"
 #include "qmoe_stream.hpp"
@@ -137,6 +138,15 @@ int linear_impl(const void* w, int fmt, int n, int k, const void* x, int xdt, in
         args.count = 1;
         args.p[0] = StreamProblem{(const uint8_t*)w, nullptr, x, y, n, k, fmt, 0, xdt, ydt, 0, 0};
         return stream_launch(args, s);
+    }
+    // two to four tokens over Q8_0 rows of up to 4096 columns: streamed once, 4x4x4 MFMA products
+    if (few_supported(fmt, w, n, k, x, xdt, tokens)) {
+        FewArgs f{};
+        f.count = 1;
+        f.tokens = tokens;
+        f.xdt = xdt;
+        f.p[0] = FewProblem{(const uint8_t*)w, x, y, n, k, ydt};
+        return few_launch(f, s);
     }
     // token batches: the token-tile GEMM (it splits K over the waves of a workgroup when the matrix
     // alone would leave most of the chip idle); the general kernel where its rules do not hold
@@ -299,20 +309,35 @@ int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stre
         dense.count = 0;
         return rc;
     };
+    FewArgs few{};
+    auto flush_few = [&]() -> int {
+        if (!few.count) return QMOE_OK;
+        const int rc = few_launch(few, (hipStream_t)stream);
+        few.count = 0;
+        return rc;
+    };
     for (int i = 0; i < count; ++i) {
         const qmoe_linear_problem& p = problems[i];
         const bool aligned = (uintptr_t)p.x % dtype_size(p.x_dtype) == 0 && (uintptr_t)p.y % dtype_size(p.y_dtype) == 0;
         const bool streams = aligned && p.tokens == 1 && stream_supported(p.fmt, p.w, p.n, p.k, p.x, p.x_dtype);
-        const bool tiles = aligned && !streams && (p.tokens >= 2 || p.fmt == QMOE_FMT_Q8_0) &&
+        const bool fews = aligned && !streams && few_supported(p.fmt, p.w, p.n, p.k, p.x, p.x_dtype, p.tokens);
+        const bool tiles = aligned && !streams && !fews && (p.tokens >= 2 || p.fmt == QMOE_FMT_Q8_0) &&
                            gemm_supported(p.fmt, p.w, 0, p.n, p.k, p.x, p.x_dtype, p.k);
         int rc;
-        if (streams) {
-            if ((rc = flush_dense())) return rc;
+        if (fews) {
+            if ((rc = flush_stream()) || (rc = flush_dense())) return rc;
+            if (few.count && (few.tokens != p.tokens || few.xdt != p.x_dtype || few.count == FEW_MAX_PROBLEMS ||
+                              few_is_wide(few.p[0].k) != few_is_wide(p.k)) && (rc = flush_few())) return rc;
+            few.tokens = p.tokens;
+            few.xdt = p.x_dtype;
+            few.p[few.count++] = FewProblem{(const uint8_t*)p.w, p.x, p.y, p.n, p.k, p.y_dtype};
+        } else if (streams) {
+            if ((rc = flush_dense()) || (rc = flush_few())) return rc;
             if (args.count && (args.p[0].fmt != p.fmt || args.count == STREAM_MAX_PROBLEMS) && (rc = flush_stream())) return rc;
             args.p[args.count++] = StreamProblem{(const uint8_t*)p.w, nullptr, p.x, p.y, p.n, p.k, p.fmt, 0,
                                                  p.x_dtype, p.y_dtype, 0, 0};
         } else if (tiles) {
-            if ((rc = flush_stream())) return rc;
+            if ((rc = flush_stream()) || (rc = flush_few())) return rc;
             if (dense.count && (dense_fmt != p.fmt || dense_xdt != p.x_dtype || dense.tokens != p.tokens ||
                                 dense.count == GEMM_MAX_PROBLEMS) && (rc = flush_dense())) return rc;
             dense_fmt = p.fmt;
@@ -320,12 +345,12 @@ int qmoe_linear_batch(const qmoe_linear_problem* problems, int count, void* stre
             dense.tokens = p.tokens;
             dense.p[dense.count++] = GemmDenseProblem{(const uint8_t*)p.w, p.x, p.y, p.n, p.k, p.y_dtype, 0};
         } else {
-            if ((rc = flush_stream()) || (rc = flush_dense())) return rc;
+            if ((rc = flush_stream()) || (rc = flush_dense()) || (rc = flush_few())) return rc;
             if ((rc = linear_impl(p.w, p.fmt, p.n, p.k, p.x, p.x_dtype, p.tokens, p.y, p.y_dtype, (hipStream_t)stream))) return rc;
         }
     }
     int rc;
-    if ((rc = flush_stream()) || (rc = flush_dense())) return rc;
+    if ((rc = flush_stream()) || (rc = flush_dense()) || (rc = flush_few())) return rc;
     return QMOE_OK;
 }
 

@@ -105,6 +105,34 @@ def test_q8_0_token_batches_ragged_rows(cuda, shape, tokens, dtype):
         assert tol <= REL_L2
 
 
+@pytest.mark.parametrize("shape", [(1030, 1024), (257, 3072), (4096, 4096), (3, 2048), (4096, 14336), (130, 8192), (66, 16384), (97, 5120)])
+@pytest.mark.parametrize("tokens,dtype", [(2, "f32"), (3, "bf16"), (4, "f32"), (4, "f16")])
+def test_q8_0_two_to_four_tokens_streamed(cuda, shape, tokens, dtype):
+    """Rows of 1024..16384 columns at 2..4 tokens take the streamed 4x4x4-MFMA kernel: every chunk
+    count of the four-wave form (up to 4096 columns), the eight-wave form with one or two chunks a
+    wave beyond, row counts that are not a multiple of four, every activation type; a batch of such
+    problems equals the separate calls bit for bit."""
+    announce("linear few tokens", shape, tokens, dtype)
+    n, k = shape
+    w = synthetic.packed_weight("Q8_0", (n, k), 411)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    xd = torch.from_numpy(synthetic.activations((tokens, k), 412, "bf16")).to(cuda).to(tdt)
+    x = xd.float().cpu().numpy()
+    want = R.linear(x, *triple(w))
+    wd = upload(w, cuda)
+    got = quantized_linear(xd, wd)
+    assert got.dtype == tdt and got.shape == (tokens, n)
+    g = got.float().cpu().numpy()
+    if dtype == "f32":
+        assert rel_l2(g, want) <= 2e-5 <= REL_L2
+    else:
+        assert np.abs(g - want).max() <= (BF16_MAX_ABS if dtype == "bf16" else 2e-3) * max(1.0, np.abs(want).max())
+    w2 = synthetic.packed_weight("Q8_0", (64, k), 413)
+    both = quantized_linear_batch([(xd, wd), (xd, upload(w2, cuda))])
+    assert torch.equal(both[0], got)
+    assert rel_l2(both[1].float().cpu().numpy(), R.linear(x, *triple(w2))) <= (2e-5 if dtype == "f32" else 5e-3)
+
+
 @pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "BF16"])
 @pytest.mark.parametrize("k", [18432, 32768])
 @pytest.mark.parametrize("tokens", [1, 3, 20])
