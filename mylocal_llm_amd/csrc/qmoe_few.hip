@@ -152,7 +152,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 4 ? FEW_NARROW_WGS : 1)) void
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const float d = h == 0 ? half_bits_to_float(r[c][0] & 0xFFFFu) : half_bits_to_float(r[c][8] >> 16);
-                float4v acc4 = {0.f, 0.f, 0.f, 0.f};
+                float4v acc4 = {0.f, 0.f, 0.f, 0.f}, low4 = {0.f, 0.f, 0.f, 0.f};   // two chains: no MFMA waits for the one before it
 #pragma unroll
                 for (int kk = 0; kk < 8; ++kk) {
                     // four codes from byte 2 + 34 h + 4 kk of the unit
@@ -166,13 +166,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES == 4 ? FEW_NARROW_WGS : 1)) void
                     ah.u[0] = x_hi[c][16 * h + 2 * kk]; ah.u[1] = x_hi[c][16 * h + 2 * kk + 1];
                     al.u[0] = x_lo[c][16 * h + 2 * kk]; al.u[1] = x_lo[c][16 * h + 2 * kk + 1];
                     acc4 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(ah.v, wb.v, acc4, 0, 0, 0);
-                    acc4 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(al.v, wb.v, acc4, 0, 0, 0);
+                    if (XDT != QMOE_DT_BF16) low4 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(al.v, wb.v, low4, 0, 0, 0);   // bf16 input has no low term
                 }
                 // a scale read from a chunk the row does not have may be anything: its sum is zero
                 // unless the scale is not finite, so such a chunk is left out
                 if (wave + WAVES * c < chunks) {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, acc4[i], acc[i]);
+                    for (int i = 0; i < 4; ++i) acc[i] = fmaf(d, XDT != QMOE_DT_BF16 ? acc4[i] + low4[i] : acc4[i], acc[i]);
                 }
             }
         }
