@@ -296,6 +296,21 @@ def moe_prefill_extra(torch, lib, device, fmt, tokens, steps, warmup):
             "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
 
 
+def layer_extra(torch, lib, device, fmt, tokens, act, steps):
+    """Eight 8B-shape layers of one format at `tokens` tokens: time per layer and weight-effective rate."""
+    s = LayerStream(torch, lib, fmt, 8, tokens, device, act=act)
+    _, m = time_steps(torch, s.step, steps, 2)
+    per_layer = m / steps / 8 * 1e-3
+    out = {"workload": f"8B projections {fmt} M={tokens} (8 layers)" + ("" if act == "f32" else f", {act} activations"),
+           "GBps": round(s.bytes_per_layer / per_layer / 1e9, 1),
+           "frac_hbm_peak": round(s.bytes_per_layer / per_layer / 1e9 / HBM_PEAK_GBS, 4),
+           "us_per_layer": round(per_layer * 1e6, 2),
+           "tokens_per_s_32_layers": round(tokens / (per_layer * 32), 1)}
+    del s
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -304,7 +319,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_layer_half"], default=None,
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_layer_half", "layer_few_tokens"], default=None,
                     help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device tensor copy (a kernel of known traffic, "
@@ -331,6 +346,9 @@ def main():
         return
     if args.only == "moe_layer_half":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, layer_half=True) for t in (1, 4)]))
+        return
+    if args.only == "layer_few_tokens":
+        print(json.dumps([layer_extra(torch, lib, device, "Q8_0", t, act, max(3, args.steps)) for t, act in ((2, "f32"), (4, "f32"), (4, "bf16"))]))
         return
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
@@ -369,20 +387,11 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_extras:
         extras = []
-        for fmt, tokens, act in (("Q6_K", 1, "f32"), ("Q5_K", 1, "f32"), ("Q4_K", 1, "f32"), ("BF16", 1, "f32"), ("Q8_0", 4, "f32"),
+        for fmt, tokens, act in (("Q6_K", 1, "f32"), ("Q5_K", 1, "f32"), ("Q4_K", 1, "f32"), ("BF16", 1, "f32"), ("Q8_0", 2, "f32"),
+                                 ("Q8_0", 4, "f32"),
                                  ("Q8_0", 16, "f32"), ("Q8_0", 64, "f32"), ("Q6_K", 16, "f32"), ("Q5_K", 16, "f32"), ("Q4_K", 16, "f32"),
-                                 ("Q8_0", 16, "bf16"), ("Q8_0", 64, "bf16"), ("Q5_K", 16, "bf16")):
-            s = LayerStream(torch, lib, fmt, 8, tokens, device, act=act)
-            w, m = time_steps(torch, s.step, max(3, args.steps // 4), 2)
-            n = max(3, args.steps // 4)
-            per_layer = m / n / 8 * 1e-3
-            extras.append({"workload": f"8B projections {fmt} M={tokens} (8 layers)" + ("" if act == "f32" else f", {act} activations"),
-                           "GBps": round(s.bytes_per_layer / per_layer / 1e9, 1),
-                           "frac_hbm_peak": round(s.bytes_per_layer / per_layer / 1e9 / HBM_PEAK_GBS, 4),
-                           "us_per_layer": round(per_layer * 1e6, 2),
-                           "tokens_per_s_32_layers": round(tokens / (per_layer * 32), 1)})
-            del s
-            torch.cuda.empty_cache()
+                                 ("Q8_0", 4, "bf16"), ("Q8_0", 16, "bf16"), ("Q8_0", 64, "bf16"), ("Q5_K", 16, "bf16")):
+            extras.append(layer_extra(torch, lib, device, fmt, tokens, act, max(3, args.steps // 4)))
         for fmt, tokens in (("Q8_0", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q6_K", 1)):
             extras.append(moe_decode_extra(torch, lib, device, fmt, tokens, max(8, args.steps), 3))
             torch.cuda.empty_cache()
