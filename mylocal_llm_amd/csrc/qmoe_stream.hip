@@ -5,7 +5,7 @@
 // unprocessed row (or group of short rows) in round-robin order that continues across
 // problem boundaries, so the HBM stream never drains between matrices; the activation
 // slice of a new problem is fetched together with that problem's first rows.
-#include "qmoe_stream.hpp"
+#include "qmoe_span.hpp"
 #include "qmoe_rowdot.hpp"
 
 namespace qmoe {
@@ -84,6 +84,7 @@ int stream_grid() {
 // Enqueue up to STREAM_MAX_PROBLEMS problems of ONE packed format -- all plain or all gate/up
 // pairs -- as one launch.  All entries must satisfy stream_supported (pairs: both matrices).
 int stream_launch(StreamArgs& args, hipStream_t s) {
+    if (span_supported(args)) return span_launch(args, s);
     const int grid = stream_grid();
     int flat = 0;   // global work items of the problems whose rows fit one wave
     int group = -1, wide_group = 1 << 20;
