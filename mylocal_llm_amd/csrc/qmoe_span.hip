@@ -83,13 +83,15 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
                      "s_load_dword %9, %10, 0x480"
                      : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9)
                      : "s"(ka) : "memory");
-        if (threadIdx.x < 2 * SPAN_MAX_KEYS + 1) ready[threadIdx.x] = 0;
+        if (threadIdx.x <= 2 * SPAN_MAX_KEYS) ready[threadIdx.x] = threadIdx.x == 2 * SPAN_MAX_KEYS ? SPAN_WAVES : 0;
         asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(t0), "+s"(t1), "+s"(t2), "+s"(t3), "+s"(t4), "+s"(t5), "+s"(t6), "+s"(t7), "+s"(t8), "+s"(t9) :: "memory");
     }
     static_assert(sizeof(SpanArgs) <= 0x500, "argument lines requested at the start");
-    __syncthreads();   // the counters are zero (nothing is in flight yet: the barrier costs no wait)
     const uint8_t* const any_w = args.p[0].w;   // a valid address for requests that carry nothing
     TR(0);
+#if defined(QMOE_SPAN_EXIT) && QMOE_SPAN_EXIT == 1
+    return;
+#endif
 #ifdef QMOE_SPAN_ICACHE_TEST
 #pragma unroll 1
     for (int rep = 0; rep < 2; ++rep) {
@@ -110,11 +112,15 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
     const uint64_t last_mask = SL::LAST_LANES >= 64 ? ~0ull : ((1ull << SL::LAST_LANES) - 1);
 
     // the next item of the workgroup, as an item of the launch
+    // The next item of the workgroup, as an item of the launch: batch b of the workgroup is batch
+    // b G + c of the launch (G workgroups), its eight items go to the waves in the order they ask.
     auto draw = [&] {
         int got = 0;
         if (lane == 0) got = (int)__atomic_fetch_add(drawn, 1u, __ATOMIC_RELAXED);   // (one lane: one item)
         const int idx = uniform(got);
-        f_g = (idx >> 3) * W + blockIdx.x * SPAN_WAVES + (idx & 7);
+        const int b = idx >> 3, pos = idx & 7;
+        const long long item = ((long long)b * gridDim.x + blockIdx.x) * SPAN_WAVES + pos;
+        f_g = item < args.items ? (int)item : args.items;
         if (f_g < args.items) queue[f_count++ & 7] = f_g;
     };
     auto next_problem = [&] {
@@ -140,7 +146,7 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
     };
     // One span into the slot at f_slot -- always SL::CHUNKS load instructions, so that the wait
     // for a span is a constant: requests that carry nothing fetch 16 bytes into a dump.
-    auto request = [&] {
+    auto issue = [&] {
         const uint8_t* m = any_w;
         int quads = 0;
         if (!f_done) {
@@ -188,19 +194,25 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
                 }
             }
         }
-        if (!f_done) {
-            f_slot = f_slot + SLOT == RING ? 0 : f_slot + SLOT;
-            if (f_parts > 1) {
-                if (++f_e < f_parts) return;
-                f_e = 0;
-            } else if (PAIR) {
-                f_m ^= 1;
-                if (f_m) return;
-            }
-            draw();
-            f_t = f_g - f_first;
-            if (f_t >= f_items) next_problem();
+    };
+    // ... and on to the span after it
+    auto advance = [&] {
+        if (f_done) return;
+        f_slot = f_slot + SLOT == RING ? 0 : f_slot + SLOT;
+        if (f_parts > 1) {
+            if (++f_e < f_parts) return;
+            f_e = 0;
+        } else if (PAIR) {
+            f_m ^= 1;
+            if (f_m) return;
         }
+        draw();
+        f_t = f_g - f_first;
+        if (f_t >= f_items) next_problem();
+    };
+    auto request = [&] {
+        issue();
+        advance();
     };
 
     // ---- activation rows ------------------------------------------------------------------------
@@ -229,7 +241,8 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
                 const float4 v = load_x4(xk.x, xk.xdt, 4 * g);
                 *(float4*)(dst + 16 * swizzled_granule(g)) = v;
             }
-            if (lane == 0) __atomic_fetch_add(&ready[key], 1u, __ATOMIC_RELAXED);
+            sig_keys |= 1u << key;   // (counted in at the next span, like the requests above)
+            sig_wait = 1;
         }
     };
     auto count_in = [&] {
@@ -248,16 +261,24 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
         for (int spins = 0; spins < (1 << 18) && *(volatile QMOE_LDS uint32_t*)counter < SPAN_WAVES; ++spins) __builtin_amdgcn_s_sleep(1);
     };
 
-    draw();
+    // The first item of every wave is fixed (item `me`), so its request and the first activation
+    // rows leave before the workgroup's waves meet; the barrier (which waits for this wave's own
+    // requests, as the first multiplication has to anyway) publishes the counters, and only then
+    // does anybody draw or count.
+    f_g = me < args.items ? me : args.items;   // (batch c of the workgroup, position `wave`)
+    if (f_g < args.items) queue[f_count++ & 7] = f_g;
     next_problem();
-#pragma unroll
-    for (int j = 0; j < PD; ++j) request();
+    issue();
     TR(1);
     int fetched = -1;  // rows 0..fetched have been requested by this wave
     x_fetch(0);
     fetched = 0;
     if (args.keys > 1) { x_fetch(1); fetched = 1; }
     TR(6);
+    __syncthreads();
+    advance();
+#pragma unroll
+    for (int j = 1; j < PD; ++j) request();
 
     // ---- multiplying side ---------------------------------------------------------------------
     uint32_t c_slot = 0;
@@ -384,12 +405,20 @@ static bool span_plan(const StreamArgs& in, SpanArgs* out) {
     SpanArgs a;
     a.count = in.count;
     a.pad = 0;
-    // The problems with the widest rows go first (their items are the largest: taken last they
-    // would leave most waves idle while a few finish), otherwise the caller's order is kept.
+    // Order: the caller's first problems with rows of up to 4096 columns that share one activation
+    // row (a small row to wait for at the start), then the problems with wider rows, widest first
+    // (their items are the largest: taken last they would leave most waves idle while a few
+    // finish), then the rest in the caller's order.
     int order[STREAM_MAX_PROBLEMS], placed = 0;
+    bool taken[STREAM_MAX_PROBLEMS] = {};
+    for (int i = 0; i < in.count && span_parts(in.p[i].k) == 1; ++i) {
+        if (i > 0 && !(in.p[i].x == in.p[i - 1].x && in.p[i].k == in.p[i - 1].k && in.p[i].xdt == in.p[i - 1].xdt)) break;
+        order[placed++] = i;
+        taken[i] = true;
+    }
     for (int parts = span_parts(STREAM_MAX_K); parts >= 1; --parts)
         for (int i = 0; i < in.count; ++i)
-            if (span_parts(in.p[i].k) == parts) order[placed++] = i;
+            if (!taken[i] && span_parts(in.p[i].k) == parts) order[placed++] = i;
     int items = 0, key = -1, prev_bytes = 0;
     for (int i = 0; i < in.count; ++i) {
         const StreamProblem& q = in.p[order[i]];

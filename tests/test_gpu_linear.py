@@ -319,3 +319,32 @@ def test_8b_projection_shapes_linearity_and_row_checks(cuda, fmt, shape):
     want = R.linear(x, *triple(sub))
     got = y.cpu().numpy()[:, rows]
     assert rel_l2(got, want) <= 3e-5  # two tokens: MFMA path, 16-bit operand splits
+
+
+LAYER_8B = [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096), (4096, 14336)]
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "Q4_K"])
+def test_full_8b_layer_in_one_batch_single_token(cuda, fmt):
+    """The benchmark's launch: the seven full-size projections of one layer through one
+    qmoe_linear_batch call at M = 1, activations shared per data-flow group (q/k/v | o | gate/up |
+    down).  Sampled rows of every problem against the oracle, the first and the last rows included;
+    a second call must give the same bits (the launch leaves no state behind)."""
+    announce("8B layer batch", fmt)
+    rng = np.random.default_rng(103)
+    xs = {name: torch.from_numpy(rng.standard_normal((1, k), dtype=np.float32)).to(cuda)
+          for name, k in (("qkv", 4096), ("o", 4096), ("gateup", 4096), ("down", 14336))}
+    groups = ["qkv", "qkv", "qkv", "o", "gateup", "gateup", "down"]
+    weights = [synthetic.packed_weight(fmt, shape, 106 + i) for i, shape in enumerate(LAYER_8B)]
+    problems = [(xs[g], upload(w, cuda)) for g, w in zip(groups, weights)]
+    outs = quantized_linear_batch(problems)
+    again = quantized_linear_batch(problems)
+    for i, (w, (n, k)) in enumerate(zip(weights, LAYER_8B)):
+        got = outs[i].cpu().numpy()
+        assert got.shape == (1, n)
+        assert np.array_equal(got.view(np.uint32), again[i].cpu().numpy().view(np.uint32))
+        rows = np.unique(np.concatenate([[0, 1, n - 2, n - 1], rng.choice(n, 40, replace=False)]))
+        sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), fmt)
+        want = R.linear(xs[groups[i]].cpu().numpy(), *triple(sub))
+        assert rel_l2(got[:, rows], want) <= 2e-6, (i, n, k)
+        assert np.isfinite(got).all()
