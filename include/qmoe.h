@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define QMOE_ABI_VERSION 2
+#define QMOE_ABI_VERSION 3
 
 /* Packed formats.  Ids 0..5 are the reference's (_FORMAT_ID,
  * mini_llm/ops/quantized_linear.py:34 and native_packed_cpu.cpp:12).  BF16 has no
@@ -187,6 +187,20 @@ size_t qmoe_moe_workspace_bytes(int tokens, int top_k, int n_experts, int d_mode
  * there is no host round trip. */
 int qmoe_moe_forward(const qmoe_moe_args* args, void* workspace, size_t workspace_bytes,
                      void* stream);
+
+/* qmoe_moe_forward for callers that cannot allocate device memory or bring a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the scratch the
+ * step needs lies in an array inside the library's device image (QMOE_MOE_STATIC_SCRATCH_BYTES,
+ * one copy per GPU, held until the process ends).  No counterpart in the reference.  Same
+ * arguments, results and errors as qmoe_moe_forward; steps that need more scratch than the
+ * array holds return QMOE_EWORKSPACE and touch nothing (the 512-expert, top-10 layer of width
+ * 2048 / 512 / 2048 fits up to 64 tokens).  The call allocates nothing, clears nothing and
+ * does not synchronise.  All calls on one GPU share the one array, which keeps the last call's
+ * contents: calls that overlap on one GPU (different streams, or threads) race and must be
+ * serialised by the caller; calls on one stream are ordered by the stream. */
+#define QMOE_MOE_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+size_t qmoe_moe_static_scratch_bytes(void);
+int qmoe_moe_forward_static(const qmoe_moe_args* args, void* stream);
 
 /* RMSNorm of the residual stream followed by the router's logits, the step in front of the MoE
  * block, in one launch:  normalized = (x * inv_rms) * gamma  with  inv_rms = 1 / sqrt(mean(x^2) + eps)

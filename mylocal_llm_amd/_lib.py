@@ -43,7 +43,7 @@ class MoeArgs(ctypes.Structure):
                 ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P)]
 
 
-ABI_VERSION = 2   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
+ABI_VERSION = 3   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
 
 _SIGNATURES = {
     "qmoe_abi_version": ([], _I),
@@ -59,6 +59,8 @@ _SIGNATURES = {
     "qmoe_moe_workspace_bytes": ([_I, _I, _I, _I, _I, _I], _SZ),
     "qmoe_moe_forward": ([ctypes.POINTER(MoeArgs), _P, _SZ, _P], _I),
     "qmoe_norm_router": ([_P, _I, _I, _P, _F, _P, _P, _I, _P, _P, _P], _I),
+    "qmoe_moe_static_scratch_bytes": ([], _SZ),
+    "qmoe_moe_forward_static": ([ctypes.POINTER(MoeArgs), _P], _I),
 }
 EXPORTS = tuple(_SIGNATURES)
 

@@ -11,6 +11,8 @@
 // with A = T*k.  Nothing is read back by the host.
 #include "qmoe_gemm.hpp"
 #include "qmoe_rowdot.hpp"
+#include <mutex>
+
 #include "qmoe_stream.hpp"
 
 namespace qmoe {
@@ -658,6 +660,51 @@ size_t qmoe_moe_workspace_bytes(int tokens, int top_k, int n_experts, int d_mode
 int qmoe_moe_forward(const qmoe_moe_args* args, void* workspace, size_t workspace_bytes, void* stream) {
     if (!args) return fail(QMOE_EINVAL, "qmoe_moe_forward: null argument struct");
     return moe_forward_impl(*args, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+// ---- the step without a caller's workspace ---------------------------------------------------------
+// Scratch for callers that cannot allocate: a file-scope array in device memory, one copy per GPU
+// the library runs on, kept until the process ends.  Its name is a host-side stand-in, not a device
+// address: the address is asked for once per device (with that device current) and only that
+// pointer is handed to the kernels.
+static constexpr size_t MOE_STATIC_SCRATCH_BYTES = QMOE_MOE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[MOE_STATIC_SCRATCH_BYTES];
+
+static int static_scratch(void** out) {
+    static constexpr int MAX_DEVICES = 64;
+    static std::mutex lock;
+    static void* per_device[MAX_DEVICES] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+        return fail(QMOE_ELAUNCH, "qmoe_moe_forward_static: no current HIP device");
+    std::lock_guard<std::mutex> guard(lock);
+    if (!per_device[dev]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(QMOE_ELAUNCH, "qmoe_moe_forward_static: scratch address: %s", hipGetErrorString(e));
+        per_device[dev] = ptr;
+    }
+    *out = per_device[dev];
+    return QMOE_OK;
+}
+
+size_t qmoe_moe_static_scratch_bytes(void) { return MOE_STATIC_SCRATCH_BYTES; }
+
+int qmoe_moe_forward_static(const qmoe_moe_args* args, void* stream) {
+    if (!args) return fail(QMOE_EINVAL, "qmoe_moe_forward_static: null argument struct");
+    const qmoe_expert_bank& b = args->bank;
+    const bool has_shared = args->shared_gate_w || args->shared_up_w || args->shared_down_w;
+    if (args->tokens > 0 && args->top_k >= 1 && b.n_experts >= 1 && b.d_model >= 1 && b.d_ff >= 1) {
+        const size_t need = moe_layout(args->tokens, args->top_k, b.n_experts, b.d_model, b.d_ff,
+                                       has_shared && args->d_ff_shared > 0 ? args->d_ff_shared : 0).total;
+        if (need > MOE_STATIC_SCRATCH_BYTES)
+            return fail(QMOE_EWORKSPACE, "qmoe_moe_forward_static: this step needs %zu bytes of scratch, the built-in area holds %zu; "
+                        "use qmoe_moe_forward with a workspace", need, MOE_STATIC_SCRATCH_BYTES);
+    }
+    void* ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    return moe_forward_impl(*args, ptr, MOE_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
 }
 
 int qmoe_grouped_decode(const float* x, const void* const* table, int n_rows, int gate_fmt, int up_fmt, int down_fmt,
