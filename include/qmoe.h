@@ -172,6 +172,13 @@ typedef struct qmoe_moe_args {
     /* optional fp32 [T, d_model]: out = residual + (routed + shared * sigmoid), the residual add
      * that follows the block (mini_llm/external/qwen3next_decoder.py:120) */
     const float* residual;
+    /* optional device word that the CALLER has set to zero: bit 0 is set when an expert id of
+     * in_ids lies outside [0, n_experts), bit 1 when one token names the same expert more than once.
+     * Such assignments contribute nothing to the output (of a repeated expert only the first slot
+     * counts); the reference's plan refuses them and leaves them to its general dispatcher
+     * (mini_llm/ops/device_expert_plan.py:17-36, :183-186).  Ids selected by the router on the device
+     * are always valid. */
+    int* status_out;
 } qmoe_moe_args;
 
 /* Bytes of workspace qmoe_moe_forward needs for these sizes (256-byte aligned). */

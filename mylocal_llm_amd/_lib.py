@@ -40,7 +40,7 @@ class MoeArgs(ctypes.Structure):
                 ("shared_gate_w", _P), ("shared_up_w", _P), ("shared_down_w", _P),
                 ("shared_gate_fmt", _I), ("shared_up_fmt", _I), ("shared_down_fmt", _I),
                 ("d_ff_shared", _I), ("shared_gate", _P),
-                ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P)]
+                ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P), ("status_out", _P)]
 
 
 ABI_VERSION = 3   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against

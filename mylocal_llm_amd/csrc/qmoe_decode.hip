@@ -34,6 +34,7 @@ struct DecodeRouteArgs {
     float* sorted_w;           // [T, k]
     float* sig;                // [T] sigmoid admission gate (1 when ungated)
     int* status;
+    int* status_out;   // the caller's word, or null
     StreamProblem* problems;   // [T * (k + 1)]
     int* problem_count;
     const void* hidden;        // [T, D]
@@ -99,17 +100,23 @@ __device__ __forceinline__ void route_token(const DecodeRouteArgs& a, int t, boo
         }
         issue();
     }
-    // rank of this selection in ascending expert id; equal ids keep slot order
+    // rank of this selection in ascending expert id; equal ids keep slot order.  An id outside the
+    // bank, or an expert the token has named in an earlier slot already, contributes nothing.
     int rank = 0;
+    bool again = false;
     for (int j = 0; j < k; ++j) {
         const int64_t other = readlane_i64(id, j);
         rank += (other < id) || (other == id && j < lane);
+        again |= other == id && j < lane;
     }
     if (lane < k) {
-        sid[rank] = id;
+        const bool in_range = id >= 0 && id < a.n_experts, ok = in_range && !again;
+        sid[rank] = ok ? id : -1;
         if (publish) {
-            const bool ok = id >= 0 && id < a.n_experts;
-            if (!ok) *a.status = 1;
+            if (!ok) {
+                const int bits = (in_range ? 0 : 1) | (again ? 2 : 0);
+                if (a.status_out) atomicOr(a.status_out, bits);
+            }
             if (a.out_weights) {
                 a.out_weights[(size_t)t * k + lane] = w;
                 a.out_ids[(size_t)t * k + lane] = id;
@@ -557,6 +564,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     r.sorted_w = w.sorted_w;
     r.sig = w.sig;
     r.status = w.status;
+    r.status_out = a.status_out;
     r.problems = (StreamProblem*)w.problems;
     r.problem_count = w.problem_count;
     r.hidden = a.hidden;

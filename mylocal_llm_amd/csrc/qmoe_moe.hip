@@ -64,6 +64,8 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
                                                                  int* __restrict__ sorted_token,
                                                                  float* __restrict__ sorted_weight,
                                                                  int* __restrict__ pos_of, int* __restrict__ status,
+                                                                 int* __restrict__ status_out,
+                                                                 float* __restrict__ out_weights, int64_t* __restrict__ out_ids,
                                                                  int* __restrict__ chunk_expert,
                                                                  int* __restrict__ chunk_start,
                                                                  int* __restrict__ chunk_count,
@@ -78,14 +80,17 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
     for (int i = tid; i < n_experts * words; i += PLAN_THREADS) selection[i] = 0u;
     if (tid == 0) *status = 0;
     __syncthreads();
-    bool bad = false;
+    // An expert id outside the bank, or the same expert named again by a token, contributes nothing
+    // (of a repeated expert the first slot counts); both are reported.
+    int bad = 0;
     for (int a = tid; a < assignments; a += PLAN_THREADS) {
         const int64_t e = ids[a];
         const int t = a / k;
-        if (e < 0 || e >= n_experts) { bad = true; continue; }
+        if (out_weights && out_weights != weights) out_weights[a] = weights[a];   // routing given by the caller: hand it back
+        if (out_ids && out_ids != ids) out_ids[a] = e;
+        if (e < 0 || e >= n_experts) { bad |= 1; continue; }
         atomicOr(&selection[(int)e * words + (t >> 5)], 1u << (t & 31));
     }
-    if (bad) *status = 1;  // out-of-range expert id: that assignment contributes nothing
     __syncthreads();
     // Per-thread chunk of consecutive experts -> counts -> two scans (sizes, non-empty flags).
     const int chunk = (n_experts + PLAN_THREADS - 1) / PLAN_THREADS;
@@ -124,6 +129,9 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
         const int64_t e64 = ids[a];
         if (e64 < 0 || e64 >= n_experts) { pos_of[a] = -1; continue; }
         const int e = (int)e64, t = a / k;
+        bool again = false;
+        for (int j = t * k; j < a; ++j) again |= ids[j] == e64;
+        if (again) { pos_of[a] = -1; bad |= 2; continue; }
         int rank = 0;
         for (int w = 0; w < (t >> 5); ++w) rank += __popc(selection[e * words + w]);
         rank += __popc(selection[e * words + (t >> 5)] & ((1u << (t & 31)) - 1u));
@@ -131,6 +139,10 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
         sorted_token[pos] = t;
         sorted_weight[pos] = weights[a];
         pos_of[a] = pos;
+    }
+    if (bad) {
+        atomicOr(status, bad);
+        if (status_out) atomicOr(status_out, bad);
     }
 }
 
@@ -231,9 +243,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
             const int q = __builtin_amdgcn_readlane(p, s);
             rank += q >= 0 && q < p;
         }
-        const int n = __popcll(__ballot(valid));
+        if (tid < 32) order[tid] = -1;   // (same wave: written before the ranked entries below)
         if (valid) order[rank] = p;
-        if (tid >= n && tid < 32) order[tid] = -1;
     }
     if (shared_out && shared_gate) {
         float a = 0.0f;
@@ -593,7 +604,8 @@ int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_b
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, s, ids, weights, a.tokens, a.top_k,
                        b.n_experts, (int*)(ws + L.offsets), (int*)(ws + L.active), (int*)(ws + L.n_active),
                        (int*)(ws + L.sorted_token), (float*)(ws + L.sorted_weight), (int*)(ws + L.pos_of),
-                       (int*)(ws + L.status), (int*)(ws + L.chunk_expert), (int*)(ws + L.chunk_start),
+                       (int*)(ws + L.status), a.status_out, a.logits ? nullptr : a.out_weights, a.logits ? nullptr : a.out_ids,
+                       (int*)(ws + L.chunk_expert), (int*)(ws + L.chunk_start),
                        (int*)(ws + L.chunk_count), (int*)(ws + L.n_chunks));
     if ((rc = check_launch("qmoe_moe_forward(plan)"))) return rc;
     const int assignments = a.tokens * a.top_k;

@@ -161,7 +161,7 @@ def norm_router(x, gamma, eps, router_weight, router_bias=None):
 
 def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared=None,
              shared_gate=None, floor=2.0 ** -14, renormalize=True, out_dtype=None,
-             return_routing=False, residual=None):
+             return_routing=False, residual=None, check_routing=False):
     """One MoE step over hidden [T, D]: routed experts (+ shared expert) -> [T, D].
 
     Routing comes from fp32 ``logits`` [T, E] (softmax/top-k on the device) or from
@@ -170,6 +170,11 @@ def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared
     admission vector (sigmoid gate).  Accumulation is fp32; the output is rounded once to
     ``out_dtype`` (default: hidden's dtype).  ``residual`` (optional fp32 [T, D]) is added to the
     block's output in the same kernels: ``residual + (routed + shared * sigmoid)``.
+
+    Precomputed ``ids`` outside ``[0, n_experts)``, or an expert repeated within one token, contribute
+    nothing (of a repeated expert the first slot counts).  With ``check_routing`` the step's status
+    word is read back afterwards (one synchronisation) and such ids raise ``ValueError``, where the
+    reference hands them to its general dispatcher (mini_llm/ops/device_expert_plan.py:183-186).
     """
     if not isinstance(hidden, torch.Tensor) or not hidden.is_cuda or hidden.dtype not in _TORCH_DTYPE_ID:
         raise TypeError("MoE hidden must be a CUDA FP16/BF16/FP32 tensor")
@@ -200,6 +205,7 @@ def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared
     step = min(t, _max_tokens_per_call(bank.n_experts))
     nbytes = lib.qmoe_moe_workspace_bytes(step, top_k, bank.n_experts, bank.d_model, bank.d_ff, f_shared)
     workspace = torch.empty(nbytes, dtype=torch.uint8, device=hidden.device)
+    status = torch.zeros(1, dtype=torch.int32, device=hidden.device) if check_routing else None
     with torch.cuda.device(hidden.device):
         for lo in range(0, t, step):
             hi = min(t, lo + step)
@@ -227,8 +233,15 @@ def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared
                 args.residual = residual[lo:hi].data_ptr()
             if return_routing:
                 args.out_weights, args.out_ids = out_w[lo:hi].data_ptr(), out_i[lo:hi].data_ptr()
+            if status is not None:
+                args.status_out = status.data_ptr()
             rc = lib.qmoe_moe_forward(ctypes.byref(args), _ptr(workspace), nbytes, _stream())
             _lib.check(rc, "Packed MoE step")
+    if status is not None:
+        bits = int(status.item())
+        if bits:
+            what = [name for bit, name in ((1, "expert ids outside the bank"), (2, "an expert repeated within a token")) if bits & bit]
+            raise ValueError("Invalid routing: " + " and ".join(what))
     return (out, out_w, out_i) if return_routing else out
 
 

@@ -426,3 +426,40 @@ def test_decode_shapes_lane_layouts_and_types(cuda, e, d, f, fsh, k, fmt, tokens
     else:
         scale = max(1.0, float(np.abs(want).max()))
         assert np.abs(out.float().cpu().numpy() - want).max() <= (2e-3 if dtype == "f16" else BF16_MAX_ABS) * scale
+
+
+@pytest.mark.parametrize("tokens", [3, 40])
+def test_invalid_routing_contributes_nothing_and_is_reported(cuda, tokens):
+    """Caller-supplied ids outside the bank, or an expert named twice by one token, contribute
+    nothing (the first slot of a repeated expert counts) on the decode launches (3 tokens) and on
+    the plan / token-batch launches (40 tokens) alike; the status word reports them.  The oracle
+    gets the same routing with the dropped assignments moved to unused experts at weight zero."""
+    announce("invalid routing", tokens)
+    e, d, f, k = 32, 256, 256, 4
+    gate, up, down, _, _ = make_layer(e, d, f, 256, ("Q8_0", "Q8_0", "Q8_0"), 510)
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 2, (tokens, d)).astype(np.float32)
+    ids = np.stack([rng.choice(24, k, replace=False) for _ in range(tokens)]).astype(np.int64)
+    w = rng.random((tokens, k)).astype(np.float32)
+    ids[0] = [5, 5, 7, 9]
+    ids[1] = [2, 40, 3, 4]
+    ids[2] = [-1, 1, 1, 6]
+    clean_ids, clean_w = ids.copy(), w.copy()
+    for t, slot, spare in ((0, 1, 24), (1, 1, 25), (2, 0, 26), (2, 2, 27)):
+        clean_ids[t, slot], clean_w[t, slot] = spare, 0.0
+
+    def expert_fn(i, rows):
+        return R.expert_ffn(rows, triple(gate.select_outer(i)), triple(up.select_outer(i)), triple(down.select_outer(i)))
+
+    want = R.experts_forward(x, clean_w, clean_ids, e, expert_fn)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    xd, wd, idd = (torch.from_numpy(a).to(cuda) for a in (x, w, ids))
+    got, back_w, back_ids = moe_step(xd, bank, k, weights=wd, ids=idd, return_routing=True)
+    assert np.isfinite(got.cpu().numpy()).all()
+    assert rel_l2(got.cpu().numpy(), want) <= 2e-5
+    # the routing the caller gave comes back as it was
+    assert np.array_equal(back_ids.cpu().numpy(), ids) and np.array_equal(back_w.cpu().numpy(), w)
+    with pytest.raises(ValueError, match="outside the bank and an expert repeated"):
+        moe_step(xd, bank, k, weights=wd, ids=idd, check_routing=True)
+    good = moe_step(xd, bank, k, weights=torch.from_numpy(clean_w).to(cuda), ids=torch.from_numpy(clean_ids).to(cuda), check_routing=True)
+    assert rel_l2(good.cpu().numpy(), want) <= 2e-5
