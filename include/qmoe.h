@@ -220,6 +220,14 @@ int qmoe_norm_router(const float* x, int tokens, int d_model, const float* gamma
                      const float* router_w, const float* router_b, int n_experts, float* normalized,
                      float* logits, void* stream);
 
+/* The router's logits alone, for a caller that holds the normalised hidden state already:
+ * logits = x @ router_w^T + router_b  (RouterInference.forward, mini_llm/ops/router_inference.py:40-46),
+ * fp32 throughout; x [T, d_model], router_w [n_experts, d_model] as stored in ffn_gate_inp,
+ * router_b fp32 [n_experts] or NULL; d_model % 4 == 0.  Same kernel and summation order as
+ * qmoe_norm_router's logits. */
+int qmoe_router_logits(const float* x, int tokens, int d_model, const float* router_w,
+                       const float* router_b, int n_experts, float* logits, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

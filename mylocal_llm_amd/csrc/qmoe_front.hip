@@ -17,7 +17,7 @@ static constexpr int FRONT_TOKENS = 8;
 
 // One expert's logits for up to NT tokens: the expert's row and gamma are read once, the tokens'
 // loads travel together.
-template <int NT>
+template <int NT, bool NORM>
 __device__ __forceinline__ void front_dots(const float* __restrict__ x, int d, int nt, const float* __restrict__ gamma,
                                            const float* __restrict__ wrow, const float* inv_rms, int lane, bool live,
                                            float bias, float* __restrict__ out, int out_stride) {
@@ -25,10 +25,16 @@ __device__ __forceinline__ void front_dots(const float* __restrict__ x, int d, i
 #pragma unroll
     for (int j = 0; j < NT; ++j) { inv[j] = inv_rms[j < nt ? j : 0]; acc[j] = 0.f; }
     for (int i = 4 * lane; i < d; i += 256) {
-        const float4 g = ldg<float4>(gamma + i), r = ldg<float4>(wrow + i);
+        const float4 r = ldg<float4>(wrow + i);
         float4 v[NT];
 #pragma unroll
         for (int j = 0; j < NT; ++j) v[j] = ldg<float4>(x + (size_t)(j < nt ? j : 0) * d + i);
+        if (!NORM) {   // x is what the router multiplies
+#pragma unroll
+            for (int j = 0; j < NT; ++j) acc[j] += (v[j].x * r.x + v[j].y * r.y) + (v[j].z * r.z + v[j].w * r.w);
+            continue;
+        }
+        const float4 g = ldg<float4>(gamma + i);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
             acc[j] += (mul_unfused(mul_unfused(v[j].x, inv[j]), g.x) * r.x + mul_unfused(mul_unfused(v[j].y, inv[j]), g.y) * r.y) +
@@ -41,6 +47,7 @@ __device__ __forceinline__ void front_dots(const float* __restrict__ x, int d, i
     }
 }
 
+template <bool NORM>
 __global__ __launch_bounds__(256) void norm_router_kernel(const float* __restrict__ x, int tokens, int d,
                                                           const float* __restrict__ gamma, float eps,
                                                           const float* __restrict__ w, const float* __restrict__ bias,
@@ -56,7 +63,7 @@ __global__ __launch_bounds__(256) void norm_router_kernel(const float* __restric
     for (int t0 = 0; t0 < tokens; t0 += FRONT_TOKENS) {
         const int nt = tokens - t0 < FRONT_TOKENS ? tokens - t0 : FRONT_TOKENS;
         __syncthreads();
-        {
+        if (NORM) {
             // sums of squares: wave w takes tokens w and w + 4 of the group, both at once
             const int ja = wave, jb = wave + 4;
             const float* xa = x + (size_t)(t0 + (ja < nt ? ja : 0)) * d;
@@ -75,10 +82,11 @@ __global__ __launch_bounds__(256) void norm_router_kernel(const float* __restric
             }
         }
         __syncthreads();
-        if (nt == 1) front_dots<1>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
-        else if (nt == 2) front_dots<2>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
-        else if (nt <= 4) front_dots<4>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
-        else front_dots<FRONT_TOKENS>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
+        if (nt == 1) front_dots<1, NORM>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
+        else if (nt == 2) front_dots<2, NORM>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
+        else if (nt <= 4) front_dots<4, NORM>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
+        else front_dots<FRONT_TOKENS, NORM>(x + (size_t)t0 * d, d, nt, gamma, wrow, inv_rms, lane, e < n_experts, bias ? bias[e < n_experts ? e : 0] : 0.0f, logits + (size_t)t0 * n_experts + e, n_experts);
+        if (!NORM) continue;
         for (int idx = threadIdx.x; idx < nt * (per_block / 4); idx += 256) {
             const int j = idx / (per_block / 4), i = c0 + 4 * (idx % (per_block / 4));
             if (i < c1) {
@@ -106,7 +114,20 @@ extern "C" int qmoe_norm_router(const float* x, int tokens, int d_model, const f
     if (d_model % 4) return fail(QMOE_EUNSUPPORTED, "qmoe_norm_router: d_model=%d is not a multiple of 4", d_model);
     if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)router_w | (uintptr_t)normalized) % 16)
         return fail(QMOE_EUNSUPPORTED, "qmoe_norm_router: x, gamma, router_w and normalized must be 16-byte aligned");
-    hipLaunchKernelGGL(norm_router_kernel, dim3((n_experts + 3) / 4), dim3(256), 0, (hipStream_t)stream, x, tokens, d_model,
+    hipLaunchKernelGGL(norm_router_kernel<true>, dim3((n_experts + 3) / 4), dim3(256), 0, (hipStream_t)stream, x, tokens, d_model,
                        gamma, eps, router_w, router_b, n_experts, normalized, logits);
     return check_launch("qmoe_norm_router");
+}
+
+extern "C" int qmoe_router_logits(const float* x, int tokens, int d_model, const float* router_w,
+                                  const float* router_b, int n_experts, float* logits, void* stream) {
+    if (!x || !router_w || !logits) return fail(QMOE_EINVAL, "qmoe_router_logits: null pointer");
+    if (tokens < 1 || d_model < 4 || n_experts < 1)
+        return fail(QMOE_EINVAL, "qmoe_router_logits: tokens=%d d_model=%d n_experts=%d", tokens, d_model, n_experts);
+    if (d_model % 4) return fail(QMOE_EUNSUPPORTED, "qmoe_router_logits: d_model=%d is not a multiple of 4", d_model);
+    if (((uintptr_t)x | (uintptr_t)router_w) % 16)
+        return fail(QMOE_EUNSUPPORTED, "qmoe_router_logits: x and router_w must be 16-byte aligned");
+    hipLaunchKernelGGL(norm_router_kernel<false>, dim3((n_experts + 3) / 4), dim3(256), 0, (hipStream_t)stream, x, tokens,
+                       d_model, (const float*)nullptr, 0.0f, router_w, router_b, n_experts, (float*)nullptr, logits);
+    return check_launch("qmoe_router_logits");
 }

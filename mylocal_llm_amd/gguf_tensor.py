@@ -1,34 +1,54 @@
-"""Decoding of individual unquantised GGUF tensors (F32 / F16 / BF16) on the host.
+"""Unquantised GGUF tensors (F32 / F16 / BF16) as host arrays.
 
-Follows mini_llm/external/gguf_tensor.py:10-51: F32 / F16 keep the reader's typed view after a
-strict shape check; BF16 arrives as bytes (or 16-bit words) and is expanded by integer shifts, so
-signed zeros and every NaN payload survive.  Quantised tensors never pass through here.
+Behaviour of mini_llm/external/gguf_tensor.py:10-51: F32 and F16 come back as the reader's own
+typed view once its shape agrees with the header; BF16 comes as raw bytes or 16-bit words and is
+widened to fp32 with integer shifts only, so signed zeros and every NaN payload survive.  Packed
+(quantised) tensors never pass through here.
 """
-import math
-
 import numpy as np
 
 
-def decode_gguf_dense(tensor):
-    """Values of ``tensor`` in canonical row-major shape (the reversed GGML shape)."""
-    kind = tensor.tensor_type.name
-    if kind not in {"F32", "F16", "BF16"}:
-        raise NotImplementedError(f"{tensor.name}: unsupported dense GGUF type {kind}")
-    shape = tuple(int(d) for d in reversed(tensor.shape))
+def canonical_shape(tensor):
+    """Row-major shape of a GGUF tensor; the file lists dimensions innermost first."""
+    return tuple(int(extent) for extent in tensor.shape)[::-1]
+
+
+def _typed_view(tensor, shape):
     values = np.asarray(tensor.data)
-    if kind != "BF16":
-        if values.shape != shape:
-            raise ValueError(f"GGUF {tensor.name}: tensor data {values.shape} != metadata {shape}")
+    if values.shape == shape:
         return values
-    if any(d <= 0 for d in shape):
+    raise ValueError(f"GGUF {tensor.name}: tensor data {values.shape} != metadata {shape}")
+
+
+def _bf16_words(tensor, payload):
+    """The payload as one flat array of little-endian 16-bit words."""
+    if payload.dtype == np.uint8:
+        return np.ascontiguousarray(payload).reshape(-1).view("<u2")
+    if payload.dtype.kind == "u" and payload.dtype.itemsize == 2:
+        return payload.reshape(-1)
+    raise ValueError(f"GGUF {tensor.name}: BF16 payload must be uint8 bytes or uint16 words, not {payload.dtype}")
+
+
+def _widen_bf16(tensor, shape):
+    if min(shape, default=1) <= 0:
         raise ValueError(f"GGUF {tensor.name}: invalid BF16 shape {shape}")
-    expected = math.prod(shape) * 2
-    if values.nbytes != expected:
-        raise ValueError(f"GGUF {tensor.name}: BF16 payload has {values.nbytes} bytes; expected {expected} for shape {shape}")
-    if values.dtype == np.dtype("uint8"):
-        words = np.ascontiguousarray(values).reshape(-1).view("<u2")
-    elif values.dtype.kind == "u" and values.dtype.itemsize == 2:
-        words = values.reshape(-1)
-    else:
-        raise ValueError(f"GGUF {tensor.name}: BF16 payload must be uint8 bytes or uint16 words, not {values.dtype}")
-    return (words.astype(np.uint32) << 16).view(np.float32).reshape(shape)
+    payload = np.asarray(tensor.data)
+    need = 2 * int(np.prod(shape, dtype=np.int64))
+    if payload.nbytes != need:
+        raise ValueError(f"GGUF {tensor.name}: BF16 payload has {payload.nbytes} bytes; expected {need} for shape {shape}")
+    wide = _bf16_words(tensor, payload).astype(np.uint32)
+    wide <<= 16
+    return wide.view(np.float32).reshape(shape)
+
+
+_DECODERS = {"F32": _typed_view, "F16": _typed_view, "BF16": _widen_bf16}
+DENSE_KINDS = frozenset(_DECODERS)
+
+
+def decode_gguf_dense(tensor):
+    """Values of ``tensor`` in canonical row-major shape."""
+    kind = tensor.tensor_type.name
+    decoder = _DECODERS.get(kind)
+    if decoder is None:
+        raise NotImplementedError(f"{tensor.name}: unsupported dense GGUF type {kind}")
+    return decoder(tensor, canonical_shape(tensor))

@@ -159,6 +159,28 @@ def norm_router(x, gamma, eps, router_weight, router_bias=None):
     return normalized, logits
 
 
+def router_logits(x, router_weight, router_bias=None):
+    """``x @ router_weight.T (+ bias)`` for fp32 ``x`` [T, D] and ``router_weight`` [E, D], on the
+    library's router kernel (RouterInference.forward, mini_llm/ops/router_inference.py:40-46)."""
+    for name, tensor in (("x", x), ("router_weight", router_weight)):
+        if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda or tensor.dtype != torch.float32 or not tensor.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous CUDA float32 tensor")
+    if x.ndim != 2 or router_weight.ndim != 2 or router_weight.shape[1] != x.shape[1] or router_weight.device != x.device:
+        raise ValueError("x [T, D] and router_weight [E, D] do not fit together")
+    t, d = x.shape
+    e = router_weight.shape[0]
+    if router_bias is not None and (router_bias.dtype != torch.float32 or tuple(router_bias.shape) != (e,) or router_bias.device != x.device):
+        raise ValueError("router_bias must be CUDA float32 [E]")
+    logits = torch.empty((t, e), dtype=torch.float32, device=x.device)
+    if t:
+        with torch.cuda.device(x.device):
+            rc = _lib.load().qmoe_router_logits(_ptr(x), t, d, _ptr(router_weight),
+                                                _ptr(router_bias) if router_bias is not None else _NULL, e,
+                                                _ptr(logits), _stream())
+        _lib.check(rc, "router logits")
+    return logits
+
+
 def moe_step(hidden, bank, top_k, *, logits=None, weights=None, ids=None, shared=None,
              shared_gate=None, floor=2.0 ** -14, renormalize=True, out_dtype=None,
              return_routing=False, residual=None, check_routing=False):
@@ -315,63 +337,8 @@ class Qwen3NextMoESpec:
 
     @classmethod
     def from_index(cls, index, layer_id):
-        from .qwen3next_gguf import _DENSE_TYPES, _GGUF_BLOCK_FORMATS, _SHARED, _meta, _positive_integer, _shape
-        if index.architecture not in ('qwen3next', 'qwen3_next'):
-            raise ValueError('Expected Qwen3-Next architecture')
-        if isinstance(layer_id, bool) or not isinstance(layer_id, int):
-            raise TypeError('layer_id must be an integer')
-        if not 0 <= layer_id < index.layers:
-            raise IndexError(f'Invalid Qwen3-Next layer {layer_id}')
-        prefix = index.architecture
-        # pruned / grouped / bias-corrected routing variants are not guessed at
-        for suffix in ('expert_weights_scale', 'expert_weights_norm', 'expert_gating_func',
-                       'expert_group_count', 'expert_group_used_count'):
-            if f'{prefix}.{suffix}' in index.reader.fields:
-                raise NotImplementedError(f'Unsupported explicit routing metadata {suffix}')
-        spec = cls(
-            _positive_integer(index.d_model, 'd_model'),
-            _positive_integer(index.d_ff, 'd_ff'),
-            _positive_integer(_meta(index.reader, f'{prefix}.expert_shared_feed_forward_length'),
-                              'expert_shared_feed_forward_length'),
-            _positive_integer(index.expert_count, 'expert_count'),
-            _positive_integer(index.experts_per_token, 'expert_used_count'),
-        )
-        explicit_ff = _meta(index.reader, f'{prefix}.expert_feed_forward_length', spec.d_ff)
-        if _positive_integer(explicit_ff, 'expert_feed_forward_length') != spec.d_ff:
-            raise ValueError('Expert width metadata disagrees with routed tensors')
-        if spec.top_k > spec.n_experts:
-            raise ValueError('expert_used_count exceeds expert_count')
-        stem = f'blk.{layer_id}.'
-        shapes = {
-            'ffn_gate_inp.weight': (spec.n_experts, spec.d_model),
-            'ffn_gate_inp_shexp.weight': (spec.d_model,),
-            'ffn_gate_shexp.weight': (spec.shared_d_ff, spec.d_model),
-            'ffn_up_shexp.weight': (spec.shared_d_ff, spec.d_model),
-            'ffn_down_shexp.weight': (spec.d_model, spec.shared_d_ff),
-            'ffn_down_exps.weight': (spec.n_experts, spec.d_model, spec.d_ff),
-        }
-        if stem + 'ffn_gate_up_exps.weight' in index.tensors:
-            shapes['ffn_gate_up_exps.weight'] = (spec.n_experts, 2 * spec.d_ff, spec.d_model)
-        else:
-            shapes['ffn_gate_exps.weight'] = (spec.n_experts, spec.d_ff, spec.d_model)
-            shapes['ffn_up_exps.weight'] = (spec.n_experts, spec.d_ff, spec.d_model)
-        for name in index.tensors:
-            if name.startswith(stem + 'ffn_') and name[len(stem):] not in shapes:
-                raise NotImplementedError(f'Unsupported FFN tensor/layout {name}')
-        for suffix, shape in shapes.items():
-            tensor = index.tensors.get(stem + suffix)
-            if tensor is None:
-                raise ValueError(f'Missing MoE tensor {stem + suffix}')
-            if _shape(tensor) != shape:
-                raise ValueError(f'{stem + suffix}: expected shape {shape}, got {_shape(tensor)}')
-            kind = tensor.tensor_type.name
-            allowed = (set(_GGUF_BLOCK_FORMATS) if '_exps.weight' in suffix else
-                       _DENSE_TYPES | set(_GGUF_BLOCK_FORMATS) if suffix in _SHARED else _DENSE_TYPES)
-            if kind not in allowed:
-                raise NotImplementedError(f'{stem + suffix}: unsupported GGUF type {kind}')
-            if kind in _GGUF_BLOCK_FORMATS and shape[-1] % _GGUF_BLOCK_FORMATS[kind][0]:
-                raise ValueError(f'{stem + suffix}: innermost dimension must be block-aligned')
-        return spec
+        from .qwen3next_gguf import check_moe_block
+        return cls(*check_moe_block(index, layer_id))
 
 
 class Qwen3NextMoEInference:
@@ -459,7 +426,7 @@ class Qwen3NextMoEInference:
             return torch.empty_like(hidden)
         b, t, d = hidden.shape
         flat = hidden.reshape(b * t, d).contiguous()
-        logits = (flat @ self.router.W_router + self.router.b_router).contiguous()
+        logits = router_logits(flat, self._router_weight)
         if self.shared_is_dense:
             # routed part on the packed kernels; shared expert and its admission gate as fp32
             # matmuls (mini_llm/external/gguf_projection.py:40-88, qwen3next_moe.py:145-147)

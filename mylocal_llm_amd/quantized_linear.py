@@ -160,6 +160,8 @@ def quantized_linear_batch(problems):
         m = x.numel() // k
         if m < 1:
             raise ValueError("Batched linear needs at least one token per problem")
+        if x.device != problems[0][0].device or weight.data.device != x.device:
+            raise ValueError("All activations and weights of a batch must live on one device")
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
         outs.append(out.reshape(tuple(x.shape[:-1]) + (n,)))
         d = descs[i]
@@ -167,7 +169,8 @@ def quantized_linear_batch(problems):
         d.fmt, d.n, d.k, d.tokens = _FORMAT_ID[weight.quant_type], n, k, m
         d.x_dtype = d.y_dtype = _TORCH_DTYPE_ID[x.dtype]
     if problems:
-        rc = _lib.load().qmoe_linear_batch(descs, len(problems), _stream())
+        with torch.cuda.device(problems[0][0].device):
+            rc = _lib.load().qmoe_linear_batch(descs, len(problems), _stream())
         _lib.check(rc, "Packed linear batch")
     return outs
 

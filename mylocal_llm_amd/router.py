@@ -78,8 +78,9 @@ class RouterInference:
             raise ValueError("normalization_floor must be finite and positive")
         self.renormalize_selected = renormalize_selected
         self.normalization_floor = float(normalization_floor)
-        self.W_router = None
+        self.W_router = None      # [d_model, n_experts], the reference's orientation
         self.b_router = None
+        self._rows = None         # (identity of W_router, its [n_experts, d_model] copy for the kernel)
 
     def route_logits(self, logits):
         """Selection and weights from precomputed logits [B, T, E] (or [T, E])."""
@@ -94,8 +95,14 @@ class RouterInference:
 
     def forward(self, x):
         batch_size, seq_len, _ = x.shape
-        x2 = x.reshape(batch_size * seq_len, self.d_model)
-        logits = x2 @ self.W_router + self.b_router
+        from .moe import router_logits
+        w = self.W_router
+        stamp = (w.data_ptr(), w._version, tuple(w.shape), w.device)
+        if self._rows is None or self._rows[0] != stamp:
+            self._rows = (stamp, w.to(torch.float32).t().contiguous())
+        x2 = x.reshape(batch_size * seq_len, self.d_model).to(torch.float32).contiguous()
+        bias = None if self.b_router is None else self.b_router.to(torch.float32).contiguous()
+        logits = router_logits(x2, self._rows[1], bias)
         logits = logits.reshape(batch_size, seq_len, self.n_experts)
         weights, ids = self.route_logits(logits)
         return weights.to(x.dtype), ids
