@@ -195,6 +195,23 @@ size_t qmoe_moe_workspace_bytes(int tokens, int top_k, int n_experts, int d_mode
 int qmoe_moe_forward(const qmoe_moe_args* args, void* workspace, size_t workspace_bytes,
                      void* stream);
 
+/* The token->expert plan alone, as qmoe_moe_forward builds it in its workspace
+ * (RoutingPlan.from_router_outputs, mini_llm/ops/routing_plan.py:52-118): the T*k assignments
+ * grouped by expert id, ascending token inside an expert.  All arrays are DEVICE memory;
+ * A = tokens * top_k.
+ *   offsets[n_experts + 1]  exclusive prefix of the per-expert assignment counts
+ *   active[n_experts]       ids of the experts with assignments, ascending (first *n_active valid)
+ *   order[A]                flat assignment index (token * top_k + slot) of each sorted position
+ *   sorted_token[A]         order / top_k;  sorted_weight[A]  weights gathered in that order
+ *   pos_of[A]               sorted position of assignment (token, slot), -1 for one that is dropped
+ *   status                  bit 0: an id outside [0, n_experts); bit 1: an expert repeated in a token
+ * Only the first offsets[n_experts] entries of the sorted arrays are written (dropped assignments
+ * shorten the list).  One workgroup builds the plan in LDS: tokens x n_experts beyond its table is
+ * QMOE_EUNSUPPORTED. */
+int qmoe_routing_plan(const int64_t* ids, const float* weights, int tokens, int top_k, int n_experts,
+                      int* offsets, int* active, int* n_active, int* order, int* sorted_token,
+                      float* sorted_weight, int* pos_of, int* status, void* stream);
+
 /* qmoe_moe_forward for callers that cannot allocate device memory or bring a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the scratch the
  * step needs lies in an array inside the library's device image (QMOE_MOE_STATIC_SCRATCH_BYTES,
@@ -227,6 +244,34 @@ int qmoe_norm_router(const float* x, int tokens, int d_model, const float* gamma
  * qmoe_norm_router's logits. */
 int qmoe_router_logits(const float* x, int tokens, int d_model, const float* router_w,
                        const float* router_b, int n_experts, float* logits, void* stream);
+
+/* ---- host twins -----------------------------------------------------------------------------
+ * The same operators over HOST pointers, computed on the CPU by one thread of scalar C++ (no
+ * stream, nothing touches the GPU).  They serve callers that hold NumPy activations and
+ * host-packed weights -- the host branch of quantized_linear
+ * (mini_llm/ops/quantized_linear.py:292-305) -- and have the argument order of the reference's
+ * native CPU backend.  Activations and results are fp32; blocks are decoded exactly as on the
+ * device, sums are fp32 in eight interleaved partials per row. */
+
+/* y[tokens, n] = x[tokens, k] @ W[n, k]^T  (mylocal_packed_gemv, native_packed_cpu.cpp:206-217). */
+int qmoe_linear_cpu(const void* w, int fmt, int n, int k, const float* x, int tokens, float* y);
+
+/* h[tokens, f] = silu(x @ G^T) * (x @ U^T)  (host branch of quantized_swiglu,
+ * mini_llm/ops/quantized_linear.py:361-368; sigmoid in the overflow-free form of
+ * native_packed_cpu.cpp:236-238). */
+int qmoe_swiglu_cpu(const void* gate, int gate_fmt, const void* up, int up_fmt, int f, int k,
+                    const float* x, int tokens, float* h);
+
+/* out[tokens, d_model] = down(swiglu(x))  (mylocal_packed_expert, native_packed_cpu.cpp:219-245). */
+int qmoe_expert_cpu(const void* gate, int gate_fmt, const void* up, int up_fmt,
+                    const void* down, int down_fmt, int d_model, int d_ff,
+                    const float* x, int tokens, float* out);
+
+/* qmoe_router_topk on the host: full softmax, exact top-k (descending logit, lower id on ties,
+ * NaN last), optional division by max(selected mass, floor)  (mini_llm/ops/router.py:21-43,
+ * mini_llm/ops/router_inference.py:47-61).  Any n, 1 <= k <= n. */
+int qmoe_router_topk_cpu(const float* logits, int tokens, int n, int k, float floor_value,
+                         int renormalize, float* weights, int64_t* ids);
 
 #ifdef __cplusplus
 }

@@ -60,6 +60,11 @@ _SIGNATURES = {
     "qmoe_moe_forward": ([ctypes.POINTER(MoeArgs), _P, _SZ, _P], _I),
     "qmoe_norm_router": ([_P, _I, _I, _P, _F, _P, _P, _I, _P, _P, _P], _I),
     "qmoe_router_logits": ([_P, _I, _I, _P, _P, _I, _P, _P], _I),
+    "qmoe_routing_plan": ([_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P], _I),
+    "qmoe_linear_cpu": ([_P, _I, _I, _I, _P, _I, _P], _I),
+    "qmoe_swiglu_cpu": ([_P, _I, _P, _I, _I, _I, _P, _I, _P], _I),
+    "qmoe_expert_cpu": ([_P, _I, _P, _I, _P, _I, _I, _I, _P, _I, _P], _I),
+    "qmoe_router_topk_cpu": ([_P, _I, _I, _I, _F, _I, _P, _P], _I),
     "qmoe_moe_static_scratch_bytes": ([], _SZ),
     "qmoe_moe_forward_static": ([ctypes.POINTER(MoeArgs), _P], _I),
 }

@@ -69,7 +69,8 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
                                                                  int* __restrict__ chunk_expert,
                                                                  int* __restrict__ chunk_start,
                                                                  int* __restrict__ chunk_count,
-                                                                 int* __restrict__ n_chunks) {
+                                                                 int* __restrict__ n_chunks,
+                                                                 int* __restrict__ order) {
     extern __shared__ uint32_t selection[];  // n_experts*words bitmap, then n_experts offsets
     __shared__ int wave_sums[PLAN_THREADS / 64];
     __shared__ int total;
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
         offsets[e] = count_prefix;
         expert_offset[e] = count_prefix;
         // the expert's assignments in chunks of GEMM_CHUNK tokens, for the token-tile GEMM
-        for (int at = 0; at < c; at += GEMM_CHUNK) {
+        for (int at = 0; chunk_expert && at < c; at += GEMM_CHUNK) {
             chunk_expert[chunk_prefix] = e;
             chunk_start[chunk_prefix] = count_prefix + at;
             chunk_count[chunk_prefix] = c - at < GEMM_CHUNK ? c - at : GEMM_CHUNK;
@@ -123,7 +124,11 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
         count_prefix += c;
         if (c > 0) active[active_prefix++] = e;
     }
-    if (tid == 0) { offsets[n_experts] = all; *n_active = all_active; *n_chunks = total; }
+    if (tid == 0) {
+        offsets[n_experts] = all;
+        *n_active = all_active;
+        if (n_chunks) *n_chunks = total;
+    }
     __syncthreads();
     for (int a = tid; a < assignments; a += PLAN_THREADS) {
         const int64_t e64 = ids[a];
@@ -139,6 +144,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void moe_plan_kernel(const int64_t* _
         sorted_token[pos] = t;
         sorted_weight[pos] = weights[a];
         pos_of[a] = pos;
+        if (order) order[pos] = a;
     }
     if (bad) {
         atomicOr(status, bad);
@@ -606,7 +612,7 @@ int moe_forward_impl(const qmoe_moe_args& a, void* workspace, size_t workspace_b
                        (int*)(ws + L.sorted_token), (float*)(ws + L.sorted_weight), (int*)(ws + L.pos_of),
                        (int*)(ws + L.status), a.status_out, a.logits ? nullptr : a.out_weights, a.logits ? nullptr : a.out_ids,
                        (int*)(ws + L.chunk_expert), (int*)(ws + L.chunk_start),
-                       (int*)(ws + L.chunk_count), (int*)(ws + L.n_chunks));
+                       (int*)(ws + L.chunk_count), (int*)(ws + L.n_chunks), (int*)nullptr);
     if ((rc = check_launch("qmoe_moe_forward(plan)"))) return rc;
     const int assignments = a.tokens * a.top_k;
     const int max_active = assignments < b.n_experts ? assignments : b.n_experts;
@@ -752,3 +758,21 @@ int qmoe_grouped_decode(const float* x, const void* const* table, int n_rows, in
 }
 
 }  // extern "C"
+
+extern "C" int qmoe_routing_plan(const int64_t* ids, const float* weights, int tokens, int top_k, int n_experts,
+                                 int* offsets, int* active, int* n_active, int* order, int* sorted_token,
+                                 float* sorted_weight, int* pos_of, int* status, void* stream) {
+    if (!ids || !weights || !offsets || !active || !n_active || !order || !sorted_token || !sorted_weight || !pos_of || !status)
+        return fail(QMOE_EINVAL, "qmoe_routing_plan: null pointer");
+    if (tokens < 1 || top_k < 1 || n_experts < 1 || top_k > n_experts || (int64_t)tokens * top_k > INT32_MAX)
+        return fail(QMOE_EINVAL, "qmoe_routing_plan: tokens=%d top_k=%d n_experts=%d", tokens, top_k, n_experts);
+    const int words = (tokens + 31) / 32;
+    const size_t plan_lds = ((size_t)n_experts * words + n_experts) * 4;
+    if (plan_lds > PLAN_LDS_LIMIT)
+        return fail(QMOE_EUNSUPPORTED, "qmoe_routing_plan: %d tokens x %d experts exceed the plan's %zu-byte table; split the batch",
+                    tokens, n_experts, PLAN_LDS_LIMIT);
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(PLAN_THREADS), plan_lds, (hipStream_t)stream, ids, weights, tokens, top_k,
+                       n_experts, offsets, active, n_active, sorted_token, sorted_weight, pos_of, status, (int*)nullptr,
+                       (float*)nullptr, (int64_t*)nullptr, (int*)nullptr, (int*)nullptr, (int*)nullptr, (int*)nullptr, order);
+    return check_launch("qmoe_routing_plan");
+}

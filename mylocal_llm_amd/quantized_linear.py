@@ -5,8 +5,10 @@ mini_llm/ops/quantized_linear.py (``quantized_linear`` :272, ``quantized_swiglu`
 ``PackedExpertFFNInference`` :403, ``DevicePackedGGUFWeight`` / ``packed_to_device``
 :45-86, ``supports_packed_gpu_type`` :36-42).  Device arrays are ``torch.Tensor`` on the
 MI355X; every operator enqueues hand-written HIP kernels of libqmoe_hip.so on torch's
-current stream through the C ABI.  There is no host/NumPy compute branch here: host
-weights must be uploaded with ``packed_to_device`` first.
+current stream through the C ABI.  NumPy activations with host ``PackedGGUFWeight`` matrices
+take the host branch of the reference (:292-305), computed by the library's scalar C++ twins;
+a device tensor never does: mixing a device activation with a host weight is an error, and the
+device path raises when the library is missing.
 """
 from dataclasses import dataclass
 import ctypes
@@ -100,9 +102,26 @@ def packed_to_device(weight, device=None):
 
 def _check_activation(x, what):
     if not isinstance(x, torch.Tensor) or not x.is_cuda:
-        raise TypeError(f"{what} must be a CUDA torch.Tensor (NumPy arrays and host weights have no path here)")
+        raise TypeError(f"{what} must be a CUDA torch.Tensor (or a NumPy array with host-packed weights)")
     if x.dtype not in _TORCH_DTYPE_ID:
         raise TypeError("GPU input must be FP16, BF16, or FP32")
+
+
+def _host_linear(x, weight, backend):
+    """NumPy activations: host-packed weight only (quantized_linear.py:292-305)."""
+    from . import native_packed_cpu
+    if x.ndim not in (2, 3):
+        raise ValueError("Expected x as [M, K] or [B, T, K]")
+    if x.shape[-1] != weight.shape[-1]:
+        raise ValueError("Input K does not match packed weight K")
+    if len(weight.shape) != 2:
+        raise ValueError("Packed linear weights must be [N, K]")
+    if not isinstance(weight, PackedGGUFWeight):
+        raise TypeError("NumPy input requires a host PackedGGUFWeight; device weights take CUDA tensors")
+    if x.dtype not in (np.float16, np.float32, np.float64):
+        raise TypeError("Reference CPU inference requires FP16/FP32/FP64 input")
+    native_packed_cpu.check_backend(backend)
+    return native_packed_cpu.packed_cpu_linear(x, weight, backend=backend)
 
 
 def quantized_linear(x, weight, *, block_k=512, cpu_packed_backend="reference"):
@@ -110,9 +129,12 @@ def quantized_linear(x, weight, *, block_k=512, cpu_packed_backend="reference"):
 
     x is a contiguous CUDA tensor [M, K] or [B, T, K] (fp16 / bf16 / fp32); the result has
     shape ``x.shape[:-1] + (N,)`` and x's dtype, accumulated in fp32 and rounded once.
-    ``block_k`` is validated as in the reference and otherwise unused;
-    ``cpu_packed_backend`` is accepted for signature compatibility only.
+    ``block_k`` is validated as in the reference and otherwise unused.  A NumPy ``x`` (fp16 /
+    fp32 / fp64) with a host ``PackedGGUFWeight`` is computed on the CPU in fp32 by the library's
+    scalar C++ (every ``cpu_packed_backend`` name selects that same code).
     """
+    if isinstance(x, np.ndarray):
+        return _host_linear(x, weight, cpu_packed_backend)
     _check_activation(x, "Packed linear input")
     if x.ndim not in (2, 3):
         raise ValueError("Expected x as [M, K] or [B, T, K]")
@@ -121,7 +143,7 @@ def quantized_linear(x, weight, *, block_k=512, cpu_packed_backend="reference"):
     if len(weight.shape) != 2:
         raise ValueError("Packed linear weights must be [N, K]")
     if isinstance(weight, PackedGGUFWeight):
-        raise TypeError("Packed host weight has no compute path here; upload it with packed_to_device")
+        raise TypeError("Packed host weight requires a NumPy input; upload it with packed_to_device for device tensors")
     if not isinstance(weight, DevicePackedGGUFWeight):
         raise TypeError("Expected PackedGGUFWeight or DevicePackedGGUFWeight")
     if not x.is_contiguous():
@@ -184,14 +206,20 @@ def quantized_swiglu(x, gate, up, *, block_k=512):
         raise TypeError("gate and up must both be host-packed or both device-packed")
     if len(gate.shape) != 2 or up.shape != gate.shape:
         raise ValueError("gate/up must share two-dimensional [F,K] shape")
-    _check_activation(x, "Quantized SwiGLU input")
+    if not isinstance(x, np.ndarray):
+        _check_activation(x, "Quantized SwiGLU input")
     if x.ndim not in (2, 3):
         raise ValueError("Expected x as [M,K] or [B,T,K]")
     f, k = gate.shape
     if x.shape[-1] != k:
         raise ValueError("Input K does not match gate/up K")
     if isinstance(gate, PackedGGUFWeight):
-        raise TypeError("Host packed gate/up have no compute path here; upload them with packed_to_device")
+        if not isinstance(x, np.ndarray):
+            raise TypeError("Host packed gate/up require NumPy activations")
+        from . import native_packed_cpu
+        return native_packed_cpu.packed_cpu_swiglu(x, gate, up)
+    if isinstance(x, np.ndarray):
+        raise TypeError("Device packed gate/up require CUDA tensors")
     if not x.is_contiguous():
         raise ValueError("GPU activations must be a contiguous tensor")
     if block_k not in (256, 512, 1024):
@@ -225,5 +253,11 @@ class PackedExpertFFNInference:
         else:
             g = quantized_linear(x, self.gate)
             u = quantized_linear(x, self.up)
-            h = (g * torch.sigmoid(g.float()).to(g.dtype)) * u
+            if isinstance(g, np.ndarray):
+                g32 = g.astype(np.float32)
+                h = ((g32 / (1.0 + np.exp(-g32))).astype(g.dtype) * u)
+            else:
+                h = (g * torch.sigmoid(g.float()).to(g.dtype)) * u
+        if isinstance(h, np.ndarray):
+            return quantized_linear(np.ascontiguousarray(h), self.down)
         return quantized_linear(h.contiguous(), self.down)

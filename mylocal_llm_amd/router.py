@@ -30,9 +30,16 @@ def _topk(logits2d, k, floor, renormalize):
 
 
 def expert_topk_forward(logits, k, output_dtype=None, return_cache=True):
-    """Full-expert softmax followed by top-k selection, without renormalisation."""
+    """Full-expert softmax followed by top-k selection, without renormalisation.  NumPy logits are
+    routed on the host by the library's scalar C++ twin, CUDA tensors by the device kernel."""
+    if isinstance(logits, np.ndarray):
+        from .native_packed_cpu import router_topk_cpu
+        weights, ids = router_topk_cpu(logits, k)
+        if output_dtype is not None and np.dtype(output_dtype) in (np.float16,):
+            weights = weights.astype(output_dtype)
+        return weights, ids, None
     if not isinstance(logits, torch.Tensor) or not logits.is_cuda:
-        raise TypeError("router logits must be a CUDA torch.Tensor")
+        raise TypeError("router logits must be a CUDA torch.Tensor or a NumPy array")
     if logits.ndim < 1 or not (1 <= int(k) <= int(logits.shape[-1])):
         raise ValueError("expert router expects 1 <= k <= n_experts")
     n = logits.shape[-1]

@@ -164,6 +164,18 @@ def test_linear_three_dimensional_input_and_shape_errors(cuda):
     with pytest.raises(TypeError, match="FP16"):
         quantized_linear(torch.zeros((2, 512), device=cuda, dtype=torch.float64), w)
     assert quantized_linear(torch.zeros((0, 512), device=cuda), w).shape == (0, 7)
+    # host and device operands do not mix: neither side is moved or dequantised behind the caller's back
+    host = synthetic.packed_weight("Q4_K", (7, 512), 1)
+    with pytest.raises(TypeError, match="NumPy input"):
+        quantized_linear(x, host)
+    with pytest.raises(TypeError, match="host PackedGGUFWeight"):
+        quantized_linear(x.cpu().numpy(), w)
+    with pytest.raises(TypeError, match="NumPy activations"):
+        quantized_swiglu(x, host, host)
+    with pytest.raises(TypeError, match="CUDA tensors"):
+        quantized_swiglu(x.cpu().numpy(), w, w)
+    # and the host twin agrees with the device kernel on the same operands
+    np.testing.assert_allclose(quantized_linear(x.cpu().numpy(), host), y.cpu().numpy(), rtol=3e-5, atol=2e-4)
 
 
 def test_linear_inputs_and_weights_are_not_mutated(cuda):
@@ -348,3 +360,57 @@ def test_full_8b_layer_in_one_batch_single_token(cuda, fmt):
         want = R.linear(xs[groups[i]].cpu().numpy(), *triple(sub))
         assert rel_l2(got[:, rows], want) <= 2e-6, (i, n, k)
         assert np.isfinite(got).all()
+
+
+@pytest.mark.parametrize("fmt,tokens", [("Q8_0", 4), ("Q8_0", 16), ("Q8_0", 64), ("Q6_K", 16), ("Q5_K", 16)])
+@pytest.mark.parametrize("shape", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)])
+def test_8b_projection_shapes_at_small_token_counts(cuda, fmt, tokens, shape):
+    """Every projection shape of the 8B layer, the wide gate/up one included, at the token counts
+    the small-batch kernels are tuned for: sampled rows (first and last among them) against the
+    oracle for every token."""
+    announce("linear 8B shape small M", fmt, tokens, shape)
+    n, k = shape
+    w = synthetic.packed_weight(fmt, (n, k), 206)
+    rng = np.random.default_rng(203)
+    x = rng.standard_normal((tokens, k), dtype=np.float32)
+    y = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    assert y.shape == (tokens, n) and np.isfinite(y).all()
+    rows = np.unique(np.concatenate([[0, 1, n - 2, n - 1], rng.choice(n, 28, replace=False)]))
+    sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), fmt)
+    assert rel_l2(y[:, rows], R.linear(x, *triple(sub))) <= 3e-5
+
+
+def test_four_host_threads_on_their_own_streams_give_identical_bits(cuda):
+    """Four threads, each on a stream of its own, twelve calls each of the single-token and the
+    small-batch linear: every result carries the bits of a single-threaded call (the reference pins
+    the same for its native backend, tests/test_0106e_cpu_packed_and_gpu_swaps.py:78-88)."""
+    import threading
+    announce("threads x streams linear")
+    w8 = upload(synthetic.packed_weight("Q8_0", (1024, 4096), 1), cuda)
+    w6 = upload(synthetic.packed_weight("Q6_K", (512, 2048), 2), cuda)
+    x1 = torch.from_numpy(synthetic.activations((1, 4096), 3)).to(cuda)
+    x16 = torch.from_numpy(synthetic.activations((16, 2048), 4)).to(cuda)
+    want1, want16 = quantized_linear(x1, w8), quantized_linear(x16, w6)
+    want_batch = quantized_linear_batch([(x1, w8), (x1, w8)])
+    torch.cuda.synchronize()
+    failures = []
+
+    def work():
+        try:
+            stream = torch.cuda.Stream(device=cuda)
+            with torch.cuda.stream(stream):
+                for _ in range(12):
+                    a, b = quantized_linear(x1, w8), quantized_linear(x16, w6)
+                    c = quantized_linear_batch([(x1, w8), (x1, w8)])
+                    stream.synchronize()
+                    if not (torch.equal(a, want1) and torch.equal(b, want16) and torch.equal(c[1], want_batch[1])):
+                        failures.append("bits differ")
+        except Exception as exc:          # surfaced below: a thread's exception is otherwise lost
+            failures.append(repr(exc))
+
+    threads = [threading.Thread(target=work) for _ in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures[:3]

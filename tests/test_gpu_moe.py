@@ -463,3 +463,104 @@ def test_invalid_routing_contributes_nothing_and_is_reported(cuda, tokens):
         moe_step(xd, bank, k, weights=wd, ids=idd, check_routing=True)
     good = moe_step(xd, bank, k, weights=torch.from_numpy(clean_w).to(cuda), ids=torch.from_numpy(clean_ids).to(cuda), check_routing=True)
     assert rel_l2(good.cpu().numpy(), want) <= 2e-5
+
+
+@pytest.mark.parametrize("tokens,zipf", [(512, 1.1), (1, None), (37, None)])
+def test_routing_plan_offsets_and_sorted_assignments_match_the_oracle(cuda, tokens, zipf):
+    """The plan the MoE step executes, read out through qmoe_routing_plan: offsets, order, sorted
+    tokens / slots / weights and active experts against RoutingPlan.from_router_outputs as the
+    oracle restates it (stable sort by expert id), on the skewed routing of the prefill
+    configuration (T = 512, Zipf 1.1, 512 experts, top-10)."""
+    from mylocal_llm_amd.routing_plan import RoutingPlan, create_routing_plan
+    announce("routing plan", tokens, zipf)
+    e, k = 512, 10
+    logits = synthetic.router_logits(tokens, e, 9, zipf=zipf) if zipf else synthetic.router_logits(tokens, e, 9)
+    w, ids = R.router_topk(logits, k, floor=2.0 ** -14)
+    plan = create_routing_plan(torch.from_numpy(ids.reshape(1, tokens, k)).to(cuda), torch.from_numpy(w.reshape(1, tokens, k)).to(cuda), k, e)
+    token, slot, order, offsets = R.routing_plan(ids, e)
+    assert plan.expert_offsets == tuple(int(v) for v in offsets)
+    assert (plan.N, plan.k, plan.n_experts) == (tokens, k, e)
+    np.testing.assert_array_equal(plan.order.cpu().numpy(), order)
+    np.testing.assert_array_equal(plan.token_indices.cpu().numpy(), token)
+    np.testing.assert_array_equal(plan.slot_indices.cpu().numpy(), slot)
+    np.testing.assert_array_equal(plan.expert_indices.cpu().numpy(), ids.reshape(-1)[order])
+    np.testing.assert_array_equal(plan.weights.cpu().numpy(), w.reshape(-1)[order])
+    counts = np.bincount(ids.reshape(-1), minlength=e)
+    assert plan.active_expert_ids() == tuple(int(i) for i in np.nonzero(counts)[0])
+    busiest = int(np.argmax(counts))
+    t_b, s_b, w_b = plan.get_expert_assignments(busiest)
+    assert plan.get_assignment_count(busiest) == counts[busiest] == len(t_b)
+    assert np.all(np.diff(t_b.cpu().numpy()) > 0)        # ascending token inside an expert
+    np.testing.assert_array_equal(ids[t_b.cpu().numpy(), s_b.cpu().numpy()], busiest)
+    # inverse map: assignment (t, slot) sits at the position the plan says
+    pos = plan.position_of_assignment.cpu().numpy().reshape(-1)
+    np.testing.assert_array_equal(order[pos], np.arange(tokens * k))
+    bad = ids.copy().reshape(1, tokens, k)
+    bad[0, 0, 0] = e
+    with pytest.raises(ValueError, match="Invalid routing"):
+        RoutingPlan.from_router_outputs(torch.from_numpy(bad).to(cuda), torch.from_numpy(w.reshape(1, tokens, k)).to(cuda), k, e)
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K"])
+@pytest.mark.parametrize("tokens", [1, 4])
+def test_decode_config_512_experts_top10_bf16_in_bf16_out(cuda, fmt, tokens):
+    """The decode configuration at full shape with bf16 hidden states in and out (the type the
+    reference's GPU runtime carries between layers): ids exact, outputs within one bf16 rounding
+    of the oracle's fp32 result."""
+    announce("moe decode full bf16", fmt, tokens)
+    e, d, f, fsh, k = 512, 2048, 512, 2048, 10
+    gate, up, down, shared, gate_vec, bank, dshared = full_layer(fmt, cuda)
+    hidden = synthetic.activations((tokens, d), 7, "bf16")
+    logits = synthetic.router_logits(tokens, e, 9)
+    hd = torch.from_numpy(hidden).to(cuda).to(torch.bfloat16)
+    out, w, ids = moe_step(hd, bank, k, logits=torch.from_numpy(logits).to(cuda), shared=dshared,
+                           shared_gate=torch.from_numpy(gate_vec).to(cuda), return_routing=True)
+    assert out.dtype == torch.bfloat16
+    want, want_w, want_ids = oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    scale = max(1.0, float(np.abs(want).max()))
+    assert np.abs(out.float().cpu().numpy() - want).max() <= BF16_MAX_ABS * scale
+    # and the same bits as the fp32 result rounded once
+    full = moe_step(torch.from_numpy(hidden).to(cuda), bank, k, logits=torch.from_numpy(logits).to(cuda), shared=dshared,
+                    shared_gate=torch.from_numpy(gate_vec).to(cuda))
+    assert torch.equal(out, full.to(torch.bfloat16))
+
+
+def test_moe_step_from_four_host_threads_on_their_own_streams(cuda):
+    """qmoe_moe_forward holds no state between calls (every call brings its workspace): four
+    threads on four streams, twelve steps each at one and at nine tokens, all bit-identical to a
+    single-threaded step."""
+    import threading
+    announce("threads x streams moe")
+    e, d, f, fsh, k = 16, 512, 256, 512, 4
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh, ("Q8_0", "Q8_0", "Q6_K"), 410)
+    bank = DevicePackedExpertBank(gate, up, down, device=cuda)
+    dshared = tuple(upload(w, cuda) for w in shared)
+    gd = torch.from_numpy(gate_vec).to(cuda)
+    cases = []
+    for tokens in (1, 9):
+        hd = torch.from_numpy(synthetic.activations((tokens, d), 7 + tokens, "bf16")).to(cuda)
+        ld = torch.from_numpy(synthetic.router_logits(tokens, e, 9 + tokens)).to(cuda)
+        cases.append((hd, ld, moe_step(hd, bank, k, logits=ld, shared=dshared, shared_gate=gd)))
+    torch.cuda.synchronize()
+    failures = []
+
+    def work():
+        try:
+            stream = torch.cuda.Stream(device=cuda)
+            with torch.cuda.stream(stream):
+                for _ in range(12):
+                    for hd, ld, want in cases:
+                        got = moe_step(hd, bank, k, logits=ld, shared=dshared, shared_gate=gd)
+                        stream.synchronize()
+                        if not torch.equal(got, want):
+                            failures.append("bits differ")
+        except Exception as exc:
+            failures.append(repr(exc))
+
+    threads = [threading.Thread(target=work) for _ in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures[:3]

@@ -127,16 +127,18 @@ def test_moe_workspace_size_is_monotone_and_aligned():
     assert lib.qmoe_moe_workspace_bytes(1, 0, 512, 2048, 512, 0) == 0
 
 
-def test_host_weights_have_no_compute_path():
+def test_host_and_device_operands_do_not_mix():
+    """NumPy activations go with host-packed weights (computed by the library's host twins);
+    nothing else is accepted in their place, and uploading needs a device."""
     torch = pytest.importorskip("torch")
     from mylocal_llm_amd.quantized_linear import quantized_linear, quantized_swiglu, packed_to_device
     w = synthetic.packed_weight("Q4_K", (2, 256), 1)
-    with pytest.raises(TypeError, match="NumPy"):
-        quantized_linear(np.zeros((2, 256), np.float32), w)
+    assert quantized_linear(np.zeros((2, 256), np.float32), w).shape == (2, 2)
+    assert quantized_swiglu(np.zeros((2, 256), np.float32), w, w).shape == (2, 2)
     with pytest.raises(TypeError, match="NumPy"):
         quantized_linear([[0] * 256], w)
-    with pytest.raises(TypeError):
-        quantized_swiglu(np.zeros((2, 256), np.float32), w, w)
+    with pytest.raises(TypeError, match="NumPy"):
+        quantized_linear(torch.zeros((2, 256)), w)      # a host tensor is not a NumPy array
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="HIP device"):
             packed_to_device(w)
