@@ -10,9 +10,13 @@ resident in HBM; tokens/s of the same stream is in `config`.
 The JSON line also carries
   roofline      achieved HBM GB/s of the dominant kernel (algorithmic bytes per launch over
                 its average launch duration, from HIP events on the launch stream)
+                and, beside it, the library's pure read kernel on the same number of bytes
+                (hbm_read_probe_GBps): what a launch of that size can stream on this device
   cpu_baseline  the NumPy restatement of the reference's packed CPU path (dequantise on every
-                call, fp32 matmul) timed on this box's host cores on a bounded sample
-  extras        other configurations (formats, token counts, MoE decode) measured the same way
+                call, fp32 matmul) timed on this box's host cores on bounded samples, with the
+                library's scalar C++ host twin, configs[0] and one MoE decode token as legs
+  extras        other configurations measured the same way: the layer launched in data-flow
+                order, other formats and token counts, MoE decode (cold rotation, and hot)
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
 """
@@ -73,7 +77,10 @@ def device_blocks(torch, fmt, n, k, gen, device):
 class LayerStream:
     """`layers` x 7 packed projections resident in HBM plus activation / output buffers."""
 
-    def __init__(self, torch, lib, fmt, layers, tokens, device, seed=106, act="f32"):
+    # projections that may run together because none reads another's output
+    GROUPS = ((0, 3), (3, 4), (4, 6), (6, 7))   # q k v | o | gate up | down
+
+    def __init__(self, torch, lib, fmt, layers, tokens, device, seed=106, act="f32", by_dependency=False):
         from mylocal_llm_amd import _lib
         self.torch, self.lib, self.fmt, self.layers, self.tokens = torch, lib, fmt, layers, tokens
         gen = torch.Generator(device=device)
@@ -98,12 +105,17 @@ class LayerStream:
                 p.w, p.x, p.y = self.weights[layer][i].data_ptr(), self.x[group[name]].data_ptr(), self.y[i].data_ptr()
                 p.fmt, p.n, p.k, p.tokens, p.x_dtype, p.y_dtype = fid, n, k, tokens, dt_id, dt_id
             self.batches.append(arr)
-        self.launches_per_step = layers  # one batched launch sequence per layer
+        self.by_dependency = by_dependency
+        self.launches_per_step = layers * (len(self.GROUPS) if by_dependency else 1)
+        stride = ctypes.sizeof(_lib.LinearProblem)
+        # (address of the first problem, count) of every ABI call of a step
+        self.calls = [(ctypes.cast(ctypes.addressof(arr) + lo * stride, ctypes.POINTER(_lib.LinearProblem)), hi - lo)
+                      for arr in self.batches for lo, hi in (self.GROUPS if by_dependency else ((0, len(PROJECTIONS)),))]
 
     def step(self, stream):
         lib = self.lib
-        for arr in self.batches:
-            rc = lib.qmoe_linear_batch(arr, len(PROJECTIONS), stream)
+        for first, count in self.calls:
+            rc = lib.qmoe_linear_batch(first, count, stream)
             if rc:
                 raise RuntimeError(lib.qmoe_last_error().decode())
 
@@ -125,39 +137,93 @@ def time_steps(torch, fn, steps, warmup):
     return wall, start.elapsed_time(stop)
 
 
-def cpu_baseline(budget_s=12.0):
-    """NumPy restatement of the reference's packed CPU path on a bounded sample of the
-    headline workload: the k and q projections of one layer (1024x4096 and 4096x4096 Q8_0,
-    M=1), dequantised on every call as the reference's default host branch does."""
+def cpu_baseline(budget_s=24.0):
+    """The reference's packed CPU path on this box's host cores, on bounded samples of the
+    benchmark's workloads.  `value` is the NumPy restatement (dequantise on every call + fp32
+    matmul, the reference's default host branch) over ALL seven projections of one 8B layer at
+    M = 1, each multiplied once; `legs` adds the same layer through the library's single-threaded
+    scalar C++ host twin on a sample, the 2048x2048 single linear of configs[0], and one token of
+    the 512-expert MoE decode step."""
     import numpy as np
     from mylocal_llm_amd import synthetic
+    from mylocal_llm_amd.native_packed_cpu import packed_cpu_linear
     from oracle import reference_np as R
-    sample = [(1024, 4096), (4096, 4096)]
-    ws = [synthetic.packed_weight("Q8_0", s, 106 + i) for i, s in enumerate(sample)]
-    x = synthetic.activations((1, 4096), 103)
-    nbytes = sum(w.nbytes for w in ws)
-    R.linear(x, ws[0].data, ws[0].shape, "Q8_0")  # warm-up
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        for w in ws:
-            R.linear(x, w.data, w.shape, "Q8_0")
-        reps += 1
-        elapsed = time.perf_counter() - t0
-        if elapsed > budget_s:
-            break
     try:
         from threadpoolctl import threadpool_info
         threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
     except Exception:
         threads = os.cpu_count() or 1
-    return {"value": round(nbytes * reps / elapsed / 1e9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
-            "sample": f"Q8_0 M=1 k-proj 1024x4096 + q-proj 4096x4096 ({nbytes} weight bytes), {reps} repetitions in "
-                      f"{elapsed:.1f}s, NumPy dequantise-every-call + fp32 matmul (oracle/reference_np.linear)",
-            "numpy": np.__version__, "host_cpus": os.cpu_count()}
+    t_begin = time.perf_counter()
+    shapes = [(n, k) for _, n, k in PROJECTIONS]
+    distinct = {}
+    for i, shape in enumerate(shapes):       # q/o and k/v, gate/up share a shape: one weight each is enough to time
+        distinct.setdefault(shape, synthetic.packed_weight("Q8_0", shape, 106 + i))
+    xs = {k: synthetic.activations((1, k), 103) for k in {k for _, k in shapes}}
+    per_shape = {}
+    for shape, w in distinct.items():
+        R.linear(xs[shape[1]], w.data, w.shape, "Q8_0")   # untimed: the first call of a size pays for fresh pages
+        t0 = time.perf_counter()
+        R.linear(xs[shape[1]], w.data, w.shape, "Q8_0")
+        per_shape[shape] = time.perf_counter() - t0
+    layer_s = sum(per_shape[shape] for shape in shapes)
+    layer_bytes = sum(weight_bytes("Q8_0", n, k) for n, k in shapes)
+    legs = []
+    # scalar C++ twin, one thread: the k projection and as many rows of the others as the budget allows
+    w = distinct[(1024, 4096)]
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 3.0:
+        packed_cpu_linear(xs[4096], w)
+        reps += 1
+    native_s = (time.perf_counter() - t0) / reps
+    legs.append({"workload": "Q8_0 M=1 k-proj 1024x4096, scalar C++ host twin (qmoe_linear_cpu)", "cores": 1, "kind": "own C++",
+                 "GBps": round(w.nbytes / native_s / 1e9, 4), "ms": round(native_s * 1e3, 3), "repetitions": reps})
+    # configs[0]: the single 2048 x 2048 Q8_0 linear at batch 1
+    w0 = synthetic.packed_weight("Q8_0", (2048, 2048), 1)
+    x0 = synthetic.activations((1, 2048), 2)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 2.0:
+        R.linear(x0, w0.data, w0.shape, "Q8_0")
+        reps += 1
+    c0_s = (time.perf_counter() - t0) / reps
+    legs.append({"workload": "configs[0]: Q8_0 2048x2048 M=1, NumPy", "cores": int(threads), "kind": "port",
+                 "GBps": round(w0.nbytes / c0_s / 1e9, 4), "ms": round(c0_s * 1e3, 3), "repetitions": reps})
+    # one token of the MoE decode step: router + 10 routed experts + shared expert (D=2048, F=512, shared 2048)
+    e, d, f, fsh, k = 512, 2048, 512, 2048, 10
+    experts = [tuple(synthetic.packed_weight("Q8_0", shape, 300 + 3 * i + j) for j, shape in enumerate(((f, d), (f, d), (d, f))))
+               for i in range(k)]
+    shared = tuple(synthetic.packed_weight("Q8_0", shape, 400 + j) for j, shape in enumerate(((fsh, d), (fsh, d), (d, fsh))))
+    hidden = synthetic.activations((1, d), 7)
+    logits = synthetic.router_logits(1, e, 9)
+    gate_vec = np.random.default_rng(1).normal(0, .02, d).astype(np.float32)
+    triple = lambda w: (w.data, w.shape, w.quant_type)
+    t0 = time.perf_counter()
+    _, ids = R.router_topk(logits, k, floor=2.0 ** -14)
+    slot_of = {int(expert): i for i, expert in enumerate(ids[0])}
+    R.moe_forward(hidden, logits, k, e, lambda i, rows: R.expert_ffn(rows, *(triple(w) for w in experts[slot_of[int(i)]])),
+                  tuple(triple(w) for w in shared), gate_vec)
+    moe_s = time.perf_counter() - t0
+    moe_bytes = sum(w.nbytes for ex in experts for w in ex) + sum(w.nbytes for w in shared)
+    legs.append({"workload": "MoE decode T=1 (512 experts, top-10, D=2048, F=512, shared 2048), NumPy", "cores": int(threads),
+                 "kind": "port", "GBps": round(moe_bytes / moe_s / 1e9, 4), "ms": round(moe_s * 1e3, 2),
+                 "tokens_per_s": round(1.0 / moe_s, 3), "repetitions": 1})
+    return {"value": round(layer_bytes / layer_s / 1e9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
+            "sample": f"one 8B layer, Q8_0, M=1: all seven projections ({layer_bytes} weight bytes) multiplied once each "
+                      f"(one warm-up and one timed call per distinct shape, {layer_s:.2f}s per layer), NumPy dequantise-every-call + fp32 matmul "
+                      "(oracle/reference_np.linear)",
+            "tokens_per_s_32_layers": round(1.0 / (32 * layer_s), 4), "legs": legs,
+            "seconds_total": round(time.perf_counter() - t_begin, 1), "numpy": np.__version__, "host_cpus": os.cpu_count()}
 
 
-def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=False):
-    """512-expert top-10 MoE decode step (D=2048, F=512, shared F=2048) over rotating banks.
+def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=False, hot=False):
+    """512-expert top-10 MoE decode step (D=2048, F=512, shared F=2048).
+
+    Cold (the default, the figure a model with dozens of layers sees): steps rotate over four
+    layers' banks, 48 different sets of router logits per bank and 48 different shared experts,
+    so an expert's bytes come round again only after several GB of other weights (far beyond the
+    4 MB L2 per XCD and the 256 MB memory-side cache).  ``hot`` repeats ONE bank, one set of
+    logits and one shared expert: everything a step reads was read by the step before.
     With ``layer_half`` a step is the second half of a decoder layer: RMSNorm + router logits of the
     fp32 residual stream in one launch, the MoE step on the normalised rows, residual added in its
     last kernel (fp32 in, fp32 out)."""
@@ -167,36 +233,38 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=
     e, d, f, fsh, k = 512, 2048, 512, 2048, 10
     gen = torch.Generator(device=device)
     gen.manual_seed(7)
-    n_banks = 4  # distinct layers' banks, so that a step never re-reads recently touched bytes
+    n_banks, n_sets, n_shared = (1, 1, 1) if hot else (4, 48, 48)
+    cycle = n_banks * n_sets
     banks, shareds = [], []
     for _ in range(n_banks):
         g = device_blocks(torch, fmt, e * f, d, gen, device)
         u = device_blocks(torch, fmt, e * f, d, gen, device)
         dn = device_blocks(torch, fmt, e * d, f, gen, device)
         banks.append(DevicePackedExpertBank((g, (e, f, d), fmt), (u, (e, f, d), fmt), (dn, (e, d, f), fmt)))
+    for _ in range(n_shared):
         shareds.append(tuple(DevicePackedGGUFWeight(device_blocks(torch, fmt, n, kk, gen, device), (n, kk), fmt)
                              for n, kk in ((fsh, d), (fsh, d), (d, fsh))))
     hidden = torch.randn((tokens, d), device=device, generator=gen).to(torch.float32 if layer_half else torch.bfloat16)
-    logits = torch.randn((n_banks, tokens, e), device=device, generator=gen)
+    logits = torch.randn((cycle, tokens, e), device=device, generator=gen)
     gate_vec = torch.randn(d, device=device, generator=gen) * 0.02
     out = torch.empty((tokens, d), device=device, dtype=hidden.dtype)
     hdt = 0 if layer_half else 2
     if layer_half:
         residual = torch.randn((tokens, d), device=device, generator=gen)
         gamma = 1 + 0.1 * torch.randn(d, device=device, generator=gen)
-        router_w = torch.randn((n_banks, e, d), device=device, generator=gen) * 0.05
+        router_w = torch.randn((cycle, e, d), device=device, generator=gen) * 0.05
     nbytes_ws = lib.qmoe_moe_workspace_bytes(tokens, k, e, d, f, fsh)
     workspace = torch.empty(nbytes_ws, dtype=torch.uint8, device=device)
     # the C ABI is the boundary: argument structs are built once, a step is one call
     calls = []
-    for i in range(n_banks):
+    for i in range(cycle):       # step i: bank i % 4, its own logits (and router matrix), shared expert i % 48
         a = _lib.MoeArgs()
         a.hidden, a.hidden_dtype, a.tokens, a.top_k = hidden.data_ptr(), hdt, tokens, k
         a.logits, a.floor_value, a.renormalize = logits[i].data_ptr(), 2.0 ** -14, 1
         if layer_half:
             a.residual = residual.data_ptr()
-        banks[i].fill(a.bank)
-        g, u, dn = shareds[i]
+        banks[i % n_banks].fill(a.bank)
+        g, u, dn = shareds[i % n_shared]
         a.shared_gate_w, a.shared_up_w, a.shared_down_w = g.data.data_ptr(), u.data.data_ptr(), dn.data.data_ptr()
         a.shared_gate_fmt = a.shared_up_fmt = a.shared_down_fmt = _lib.FORMAT_ID[fmt]
         a.d_ff_shared, a.shared_gate = fsh, gate_vec.data_ptr()
@@ -206,10 +274,10 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=
     wsp = ctypes.c_void_p(workspace.data_ptr())
 
     def fn(stream):
-        i = state["i"] % n_banks
+        i = state["i"] % cycle
         a = calls[i]
         state["i"] += 1
-        if layer_half:  # normalised rows -> `hidden`, logits -> this bank's logits buffer
+        if layer_half:  # normalised rows -> `hidden`, logits -> this step's logits buffer
             rc = lib.qmoe_norm_router(residual.data_ptr(), tokens, d, gamma.data_ptr(), 1e-6, router_w[i].data_ptr(), None, e,
                                       hidden.data_ptr(), logits[i].data_ptr(), stream)
             if rc:
@@ -219,14 +287,18 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=
             raise RuntimeError(lib.qmoe_last_error().decode())
 
     wall, ms = time_steps(torch, fn, steps, warmup)
-    # algorithmic bytes: distinct selected experts (averaged over the banks' logits) + shared expert
-    ids = torch.topk(logits, k, dim=-1).indices
-    distinct = sum(len(torch.unique(ids[i])) for i in range(n_banks)) / n_banks
+    # algorithmic bytes: distinct selected experts (averaged over the steps actually run) + shared expert
+    used = sorted({j % cycle for j in range(warmup, warmup + steps)})
+    ids = torch.topk(logits[used], k, dim=-1).indices
+    distinct = sum(len(torch.unique(ids[j])) for j in range(len(used))) / len(used)
     eb = 3 * weight_bytes(fmt, f, d)
     sb = 3 * weight_bytes(fmt, fsh, d)
     nbytes = distinct * eb + sb + (e * d * 4 if layer_half else 0)
     per_step = ms / steps * 1e-3
-    return {"workload": f"moe_{'layer_half' if layer_half else 'decode'}_{fmt}_T{tokens}", "ms_per_step": round(ms / steps, 4),
+    return {"workload": f"moe_{'layer_half' if layer_half else 'decode'}_{fmt}_T{tokens}" + ("_hot" if hot else ""),
+            "residency": "hot: one bank, one set of logits, every step re-reads the bytes of the step before" if hot else
+                         "cold: 4 banks x 48 logits sets x 48 shared experts in rotation",
+            "ms_per_step": round(ms / steps, 4),
             "weight_bytes": int(nbytes), "distinct_experts": distinct,
             "GBps": round(nbytes / per_step / 1e9, 1), "frac_hbm_peak": round(nbytes / per_step / 1e9 / HBM_PEAK_GBS, 4),
             "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
@@ -296,12 +368,36 @@ def moe_prefill_extra(torch, lib, device, fmt, tokens, steps, warmup):
             "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
 
 
-def layer_extra(torch, lib, device, fmt, tokens, act, steps):
-    """Eight 8B-shape layers of one format at `tokens` tokens: time per layer and weight-effective rate."""
-    s = LayerStream(torch, lib, fmt, 8, tokens, device, act=act)
+def read_probe_extra(torch, lib, device, nbytes, steps, warmup=3):
+    """The library's pure read kernel over eight rotating buffers of `nbytes` each: the streaming
+    ceiling of this device for launches the size of one layer."""
+    nbytes = nbytes // 4096 * 4096
+    buffers = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=device) for _ in range(8)]
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    state = {"i": 0}
+
+    def fn(stream):
+        buf = buffers[state["i"] % len(buffers)]
+        state["i"] += 1
+        rc = lib.qmoe_read_probe(buf.data_ptr(), nbytes, 0x12345678, sink.data_ptr(), stream)
+        if rc:
+            raise RuntimeError(lib.qmoe_last_error().decode())
+
+    _, ms = time_steps(torch, fn, steps, warmup)
+    per_launch = ms / steps * 1e-3
+    return {"workload": f"hbm_read_probe {nbytes} bytes per launch (qmoe_read_probe, 8 rotating buffers)",
+            "GBps": round(nbytes / per_launch / 1e9, 1), "frac_hbm_peak": round(nbytes / per_launch / 1e9 / HBM_PEAK_GBS, 4),
+            "us_per_launch": round(per_launch * 1e6, 2)}
+
+
+def layer_extra(torch, lib, device, fmt, tokens, act, steps, by_dependency=False):
+    """Eight 8B-shape layers of one format at `tokens` tokens: time per layer and weight-effective rate.
+    ``by_dependency`` launches what a decoder can launch: q k v | o | gate up | down, four calls per layer."""
+    s = LayerStream(torch, lib, fmt, 8, tokens, device, act=act, by_dependency=by_dependency)
     _, m = time_steps(torch, s.step, steps, 2)
     per_layer = m / steps / 8 * 1e-3
-    out = {"workload": f"8B projections {fmt} M={tokens} (8 layers)" + ("" if act == "f32" else f", {act} activations"),
+    out = {"workload": f"8B projections {fmt} M={tokens} (8 layers)" + ("" if act == "f32" else f", {act} activations")
+                       + (", four launches per layer in data-flow order (q k v | o | gate up | down)" if by_dependency else ""),
            "GBps": round(s.bytes_per_layer / per_layer / 1e9, 1),
            "frac_hbm_peak": round(s.bytes_per_layer / per_layer / 1e9 / HBM_PEAK_GBS, 4),
            "us_per_layer": round(per_layer * 1e6, 2),
@@ -319,7 +415,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_layer_half", "layer_few_tokens"], default=None,
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_layer_half", "layer_few_tokens", "read_probe",
+                                       "layer_q6_k", "layer_q5_k", "layer_q4_k", "layer_by_dependency"], default=None,
                     help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device tensor copy (a kernel of known traffic, "
@@ -344,6 +441,19 @@ def main():
     if args.only == "moe_decode":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup) for t in (1, 4, 16)]))
         return
+    if args.only == "moe_decode_hot":
+        print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, hot=True) for t in (1, 4, 16)]))
+        return
+    if args.only == "read_probe":
+        layer_bytes = sum(weight_bytes("Q8_0", n, k) for _, n, k in PROJECTIONS)
+        print(json.dumps([read_probe_extra(torch, lib, device, b, max(50, args.steps)) for b in (layer_bytes, 1 << 30)]))
+        return
+    if args.only in ("layer_q6_k", "layer_q5_k", "layer_q4_k"):
+        print(json.dumps(layer_extra(torch, lib, device, args.only[6:].upper(), 1, "f32", max(10, args.steps))))
+        return
+    if args.only == "layer_by_dependency":
+        print(json.dumps(layer_extra(torch, lib, device, "Q8_0", 1, "f32", max(10, args.steps), by_dependency=True)))
+        return
     if args.only == "moe_layer_half":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, layer_half=True) for t in (1, 4)]))
         return
@@ -364,11 +474,12 @@ def main():
     launches = args.steps * stream.launches_per_step
     launch_ms = ms / launches
     achieved = stream.bytes_per_layer / (launch_ms * 1e-3) / 1e9
-    traffic = None
+    traffic = traffic_source = None
     traffic_file = os.path.join(ROOT, "profiles", "stream_q8_0_layer_m1_hbm_traffic.json")
     if os.path.exists(traffic_file):  # from the two rocprofv3 --pmc runs described beside that file
         with open(traffic_file) as fh:
             traffic = json.load(fh).get("traffic_bytes_per_launch")
+        traffic_source = "from profiles/stream_q8_0_layer_m1_hbm_traffic.json (two rocprofv3 --pmc runs of this command, not measured in this run)"
     result = {
         "metric": "effective weight GB/s (Q8_0 8B projections, M=1, 32 layers streamed)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -377,16 +488,23 @@ def main():
         "config": {"workload": f"configs[1]: Llama-3-8B-shaped Q8_0 projections, M=1, {args.layers} layers x 7 "
                                "projections streamed back-to-back, one batched launch sequence per layer",
                    "weight_bytes_per_step": total_bytes, "tokens_per_s": round(1.0 / step_s, 1),
+                   "tokens_per_s_is": "projection-only (no attention, norms or sampling), one launch per layer: the seven "
+                                      "projections of a layer are multiplied together although o, gate/up and down depend on "
+                                      "each other in a decoder; the data-flow-ordered figure is the first entry of extras",
                    "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4), "activations": "fp32 N(0,1)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "linear (Q8_0, M=1), one layer = 7 projections per launch sequence",
                      "bytes_per_launch": stream.bytes_per_layer, "avg_launch_us": round(launch_ms * 1e3, 3)},
     }
     del stream
     torch.cuda.empty_cache()
+    probe = read_probe_extra(torch, lib, device, result["roofline"]["bytes_per_launch"], 64)
+    result["roofline"]["hbm_read_probe_GBps"] = probe["GBps"]
+    result["roofline"]["frac_of_read_probe"] = round(achieved / probe["GBps"], 4)
+    torch.cuda.empty_cache()
     if not args.no_extras:
-        extras = []
+        extras = [layer_extra(torch, lib, device, "Q8_0", 1, "f32", max(3, args.steps // 4), by_dependency=True)]
         for fmt, tokens, act in (("Q6_K", 1, "f32"), ("Q5_K", 1, "f32"), ("Q4_K", 1, "f32"), ("BF16", 1, "f32"), ("Q8_0", 2, "f32"),
                                  ("Q8_0", 4, "f32"),
                                  ("Q8_0", 16, "f32"), ("Q8_0", 64, "f32"), ("Q6_K", 16, "f32"), ("Q5_K", 16, "f32"), ("Q4_K", 16, "f32"),
@@ -395,6 +513,8 @@ def main():
         for fmt, tokens in (("Q8_0", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q6_K", 1)):
             extras.append(moe_decode_extra(torch, lib, device, fmt, tokens, max(8, args.steps), 3))
             torch.cuda.empty_cache()
+        extras.append(moe_decode_extra(torch, lib, device, "Q8_0", 1, max(8, args.steps), 3, hot=True))
+        torch.cuda.empty_cache()
         for tokens in (1, 4):
             extras.append(moe_decode_extra(torch, lib, device, "Q8_0", tokens, max(8, args.steps), 3, layer_half=True))
             torch.cuda.empty_cache()

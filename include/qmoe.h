@@ -245,6 +245,12 @@ int qmoe_norm_router(const float* x, int tokens, int d_model, const float* gamma
 int qmoe_router_logits(const float* x, int tokens, int d_model, const float* router_w,
                        const float* router_b, int n_experts, float* logits, void* stream);
 
+/* Measurement aid, no counterpart in the reference: reads `bytes` (a multiple of 4096) of device
+ * memory once with 16-byte loads, one workgroup of eight waves per CU, and writes nothing unless
+ * the XOR of all dwords equals `match` (then that value goes to sink[0]).  Its duration is the
+ * streaming-read ceiling of the device for a launch of that size. */
+int qmoe_read_probe(const void* buffer, size_t bytes, uint32_t match, uint32_t* sink, void* stream);
+
 /* ---- host twins -----------------------------------------------------------------------------
  * The same operators over HOST pointers, computed on the CPU by one thread of scalar C++ (no
  * stream, nothing touches the GPU).  They serve callers that hold NumPy activations and

@@ -61,6 +61,7 @@ _SIGNATURES = {
     "qmoe_norm_router": ([_P, _I, _I, _P, _F, _P, _P, _I, _P, _P, _P], _I),
     "qmoe_router_logits": ([_P, _I, _I, _P, _P, _I, _P, _P], _I),
     "qmoe_routing_plan": ([_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P], _I),
+    "qmoe_read_probe": ([_P, _SZ, ctypes.c_uint32, _P, _P], _I),
     "qmoe_linear_cpu": ([_P, _I, _I, _I, _P, _I, _P], _I),
     "qmoe_swiglu_cpu": ([_P, _I, _P, _I, _I, _I, _P, _I, _P], _I),
     "qmoe_expert_cpu": ([_P, _I, _P, _I, _P, _I, _I, _I, _P, _I, _P], _I),

@@ -20,13 +20,6 @@ namespace qmoe {
 #define QMOE_LDS __attribute__((address_space(3)))
 typedef QMOE_LDS uint32_t* lds_counter;
 
-#ifdef QMOE_SPAN_TRACE
-__device__ unsigned long long* g_trace;
-#define TR(i) do { if ((threadIdx.x & 63) == 0) g_trace[((size_t)blockIdx.x * SPAN_WAVES + (threadIdx.x >> 6)) * 16 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define TR(i)
-#endif
-
 // Activations in LDS as fp32: 16-byte granules XOR-swizzled inside groups of 16 64-element units,
 // so that lanes reading granule i of consecutive units hit different banks without padding.
 // The map is its own inverse.
@@ -88,19 +81,6 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
     }
     static_assert(sizeof(SpanArgs) <= 0x500, "argument lines requested at the start");
     const uint8_t* const any_w = args.p[0].w;   // a valid address for requests that carry nothing
-    TR(0);
-#if defined(QMOE_SPAN_EXIT) && QMOE_SPAN_EXIT == 1
-    return;
-#endif
-#ifdef QMOE_SPAN_ICACHE_TEST
-#pragma unroll 1
-    for (int rep = 0; rep < 2; ++rep) {
-        const unsigned long long a = __builtin_readcyclecounter();
-        asm volatile(".rept 1024\n\ts_nop 0\n\t.endr" ::: "memory");
-        const unsigned long long b = __builtin_readcyclecounter();
-        if (lane == 0) g_trace[((size_t)blockIdx.x * SPAN_WAVES + wave) * 16 + 10 + rep] = b - a;
-    }
-#endif
 
     // ---- request side -----------------------------------------------------------------------
     int f_pi = -1, f_t = 0, f_items = 0, f_first = 0, f_g = 0, f_count = 0, f_e = 0, f_parts = 1, f_rpi = 1, f_n = 0, f_k = 256, f_m = 0;
@@ -224,11 +204,7 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
         uint8_t* const dst = xs + xk.offset;
         if (xk.xdt == QMOE_DT_F32) {
             const uint8_t* const src = (const uint8_t*)xk.x;
-#ifdef QMOE_SPAN_NOX
-            for (int c = wave; c < 0; c += SPAN_WAVES) {
-#else
             for (int c = wave; c < chunks; c += SPAN_WAVES) {
-#endif
                 set_m0((uint32_t)(uintptr_t)dst + 1024 * c);
                 const uint32_t o = 16 * swizzled_granule(lane + 64 * c);
                 QMOE_DMA16(src, o, 0);
@@ -269,12 +245,10 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
     if (f_g < args.items) queue[f_count++ & 7] = f_g;
     next_problem();
     issue();
-    TR(1);
     int fetched = -1;  // rows 0..fetched have been requested by this wave
     x_fetch(0);
     fetched = 0;
     if (args.keys > 1) { x_fetch(1); fetched = 1; }
-    TR(6);
     __syncthreads();
     advance();
 #pragma unroll
@@ -293,7 +267,6 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
     int cur_key = -1, sliced_key = -1;
     const uint8_t* xrow = xs;
     float xr[64], aux[8];
-    bool first_wait = true;
     for (int pi = 0; pi < args.count; ++pi) {
         const SpanProblem& p = args.p[pi];
         const int key = p.key;
@@ -307,13 +280,11 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
             }
             if (sig_keys) {
                 wait_vmcnt<0>();
-                if (first_wait) TR(7);
-                count_in();
+                                count_in();
             }
             spin_until(&ready[key]);
             xrow = xs + args.key[key].offset;
-            if (first_wait) TR(2);
-        }
+                    }
         const int first = p.first_item, end = p.end_item;
         if (c_g >= end) continue;
         const int k = p.k, n = p.n, units = k >> 6, ydt = p.ydt;
@@ -332,15 +303,13 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
             if (sliced_key != key) {
                 U::load_x(SwizzledX{xrow}, active ? u : 0, xr, aux);
                 sliced_key = key;
-                if (first_wait) TR(8);
-            }
+                            }
             const uint32_t lane_off = sub * ((k >> 8) * S::PP4 * 16) + S::unit_offset(active ? u : 0);
             for (; c_g < end; c_next()) {
                 const int t = c_g - first;
                 if (fetched == key) look_ahead();
                 request();
                 arrive();
-                if (first_wait) { TR(3); first_wait = false; }
                 uint32_t r[U::RAW];
                 S::read(ring + c_slot + lane_off, u, r);
                 float v = U::dot(r, xr, aux);
@@ -376,7 +345,6 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
                     const bool active = u < units;
                     U::load_x(SwizzledX{xrow}, active ? u : 0, xr, aux);
                     arrive();
-                    if (first_wait) { TR(3); first_wait = false; }
                     uint32_t r[U::RAW];
                     S::read(ring + c_slot + lane_off, lane, r);
                     const float d = U::dot(r, xr, aux);
@@ -391,7 +359,6 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
     }
     if (cur_key >= 0 && lane == 0) __atomic_fetch_add(&left[cur_key], 1u, __ATOMIC_RELAXED);
     wait_vmcnt<0>();
-    TR(4);
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -469,50 +436,7 @@ static int span_launch_as(const SpanArgs& args, hipStream_t s) {
         configured = true;
     }
     const int grid = stream_grid() / 2;   // one workgroup per CU
-#ifdef QMOE_SPAN_TRACE
-    static unsigned long long* buf = nullptr;
-    static int calls = 0;
-    const size_t words = (size_t)grid * SPAN_WAVES * 16;
-    if (!buf) {
-        hipMalloc(&buf, words * 8);
-        hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &buf, sizeof(buf));
-    }
-    hipMemsetAsync(buf, 0, words * 8, s);
-#endif
     hipLaunchKernelGGL((span_kernel<FMT, PAIR, PD>), dim3(grid), dim3(SPAN_THREADS), lds, s, args);
-#ifdef QMOE_SPAN_TRACE
-    if (++calls == 40) {
-        hipStreamSynchronize(s);
-        unsigned long long* h = (unsigned long long*)malloc(words * 8);
-        hipMemcpy(h, buf, words * 8, hipMemcpyDeviceToHost);
-        const int waves = grid * SPAN_WAVES;
-        unsigned long long t0 = ~0ull;
-        for (int w = 0; w < waves; ++w) if (h[w * 16] && h[w * 16] < t0) t0 = h[w * 16];
-        const char* names[] = {"entry", "first requests out", "activations there (first row)", "first data", "end", "after barrier", "x requested", "own x + first item arrived", "slice read issued"};
-        for (int i = 0; i < 9; ++i) {
-            double mn = 1e18, mx = 0, sum = 0; int n = 0;
-            for (int w = 0; w < waves; ++w) { if (!h[w * 16 + i]) continue; const double v = (double)(h[w * 16 + i] - t0) * 0.01; mn = v < mn ? v : mn; mx = v > mx ? v : mx; sum += v; ++n; }
-            fprintf(stderr, "trace %-20s n=%d min %.2f avg %.2f max %.2f us\n", names[i], n, mn, n ? sum / n : 0, mx);
-        }
-        double byx[8] = {0}, mxx[8] = {0};
-        for (int c = 0; c < grid; ++c)
-            for (int w = 0; w < SPAN_WAVES; ++w) {
-                const double e = (double)(h[((size_t)c * SPAN_WAVES + w) * 16 + 4] - t0) * 0.01;
-                byx[c % 8] += e / (grid / 8 * SPAN_WAVES); mxx[c % 8] = e > mxx[c % 8] ? e : mxx[c % 8];
-            }
-#ifdef QMOE_SPAN_ICACHE_TEST
-        for (int rep = 0; rep < 2; ++rep) { double sm = 0, mx = 0; for (int w = 0; w < waves; ++w) { const double v = (double)h[w * 16 + 10 + rep]; sm += v / waves; mx = v > mx ? v : mx; } fprintf(stderr, "trace 1024 s_nop (4 KB of code), pass %d: avg %.0f max %.0f clocks\n", rep, sm, mx); }
-#endif
-        for (int x = 0; x < 8; ++x) fprintf(stderr, "trace workgroups %d mod 8: end avg %.2f max %.2f\n", x, byx[x], mxx[x]);
-        for (int w = 0; w < SPAN_WAVES; ++w) {
-            double e = 0, mx = 0, mn = 1e9, fd = 0;
-            for (int c = 0; c < grid; ++c) { const unsigned long long* t = h + ((size_t)c * SPAN_WAVES + w) * 16; const double v = (double)(t[4] - t0) * 0.01; e += v / grid; mx = v > mx ? v : mx; mn = v < mn ? v : mn; fd += (double)(t[3] - t0) * 0.01 / grid; }
-            fprintf(stderr, "trace wave %d of its workgroup: first data avg %.2f end min %.2f avg %.2f max %.2f\n", w, fd, mn, e, mx);
-        }
-        for (int c = 0; c < 3; ++c) { fprintf(stderr, "wg %d ends:", c * 37); for (int w = 0; w < SPAN_WAVES; ++w) fprintf(stderr, " %.1f", (double)(h[((size_t)c * 37 * SPAN_WAVES + w) * 16 + 4] - t0) * 0.01); fprintf(stderr, "\n"); }
-        free(h);
-    }
-#endif
     return check_launch("span kernel");
 }
 
@@ -539,11 +463,7 @@ bool span_supported(const StreamArgs& args) {
 int span_launch(const StreamArgs& in, hipStream_t s) {
     const bool pair = in.p[0].w2 != nullptr;
     switch (in.p[0].fmt) {
-#ifdef QMOE_SPAN_Q8PD
-    case QMOE_FMT_Q8_0: return span_launch_fmt<QMOE_FMT_Q8_0, QMOE_SPAN_Q8PD>(in, pair, s);
-#else
     case QMOE_FMT_Q8_0: return span_launch_fmt<QMOE_FMT_Q8_0, 2>(in, pair, s);
-#endif
     case QMOE_FMT_Q6_K: return span_launch_fmt<QMOE_FMT_Q6_K, 2>(in, pair, s);
     case QMOE_FMT_Q5_K: return span_launch_fmt<QMOE_FMT_Q5_K, 3>(in, pair, s);
     default: return span_launch_fmt<QMOE_FMT_Q4_K, 3>(in, pair, s);
