@@ -259,6 +259,10 @@ int qmoe_read_probe(const void* buffer, size_t bytes, uint32_t match, uint32_t* 
  * native CPU backend.  Activations and results are fp32; blocks are decoded exactly as on the
  * device, sums are fp32 in eight interleaved partials per row. */
 
+/* out[n*k] fp32 = dequantised packed matrix on the host, the values of qmoe_dequantize bit for bit
+ * (PackedGGUFWeight.dequantize_reference, mini_llm/ops/quantized_weight.py:151-250). */
+int qmoe_dequantize_cpu(const void* w, int fmt, int64_t n, int64_t k, float* out);
+
 /* y[tokens, n] = x[tokens, k] @ W[n, k]^T  (mylocal_packed_gemv, native_packed_cpu.cpp:206-217). */
 int qmoe_linear_cpu(const void* w, int fmt, int n, int k, const float* x, int tokens, float* y);
 

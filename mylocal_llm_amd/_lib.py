@@ -62,6 +62,7 @@ _SIGNATURES = {
     "qmoe_router_logits": ([_P, _I, _I, _P, _P, _I, _P, _P], _I),
     "qmoe_routing_plan": ([_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P], _I),
     "qmoe_read_probe": ([_P, _SZ, ctypes.c_uint32, _P, _P], _I),
+    "qmoe_dequantize_cpu": ([_P, _I, _I64, _I64, _P], _I),
     "qmoe_linear_cpu": ([_P, _I, _I, _I, _P, _I, _P], _I),
     "qmoe_swiglu_cpu": ([_P, _I, _P, _I, _I, _I, _P, _I, _P], _I),
     "qmoe_expert_cpu": ([_P, _I, _P, _I, _P, _I, _I, _I, _P, _I, _P], _I),

@@ -96,6 +96,17 @@ void decode_q6_k(const uint8_t* b, float* w) {
     }
 }
 
+void decode_block(int fmt, const uint8_t* block, float* w) {
+    switch (fmt) {
+    case QMOE_FMT_Q8_0: decode_q8_0(block, w); break;
+    case QMOE_FMT_Q4_0: decode_q4_0(block, w); break;
+    case QMOE_FMT_Q4_K: decode_q45_k<false>(block, w); break;
+    case QMOE_FMT_Q5_K: decode_q45_k<true>(block, w); break;
+    case QMOE_FMT_Q3_K: decode_q3_k(block, w); break;
+    default: decode_q6_k(block, w); break;
+    }
+}
+
 // One packed row times one activation row.
 float row_dot(const uint8_t* row, int fmt, int k, const float* x) {
     float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -105,14 +116,7 @@ float row_dot(const uint8_t* row, int fmt, int k, const float* x) {
         const int elems = block_elems(fmt), bytes = block_bytes(fmt);
         float w[256];
         for (int at = 0; at < k; at += elems, row += bytes) {
-            switch (fmt) {
-            case QMOE_FMT_Q8_0: decode_q8_0(row, w); break;
-            case QMOE_FMT_Q4_0: decode_q4_0(row, w); break;
-            case QMOE_FMT_Q4_K: decode_q45_k<false>(row, w); break;
-            case QMOE_FMT_Q5_K: decode_q45_k<true>(row, w); break;
-            case QMOE_FMT_Q3_K: decode_q3_k(row, w); break;
-            default: decode_q6_k(row, w); break;
-            }
+            decode_block(fmt, row, w);
             for (int i = 0; i < elems; ++i) part[i & 7] += w[i] * x[at + i];
         }
     }
@@ -139,6 +143,21 @@ inline uint32_t selection_key(float v) {
 }
 
 }  // namespace
+
+extern "C" int qmoe_dequantize_cpu(const void* w, int fmt, int64_t n, int64_t k, float* out) {
+    if (!w || !out) return fail(QMOE_EINVAL, "qmoe_dequantize_cpu: null pointer");
+    if (!format_implemented(fmt)) return fail(QMOE_EUNSUPPORTED, "qmoe_dequantize_cpu: format %d", fmt);
+    if (n < 1 || k < 1 || k % block_elems(fmt)) return fail(QMOE_EINVAL, "qmoe_dequantize_cpu: n=%lld k=%lld", (long long)n, (long long)k);
+    const int elems = block_elems(fmt), bytes = block_bytes(fmt);
+    const uint8_t* block = (const uint8_t*)w;
+    const int64_t blocks = n * (k / elems);
+    if (fmt == QMOE_FMT_BF16) {
+        for (int64_t i = 0; i < blocks; ++i) out[i] = bits_to_float((uint32_t)u16_at(block + 2 * i) << 16);
+        return QMOE_OK;
+    }
+    for (int64_t i = 0; i < blocks; ++i, block += bytes, out += elems) decode_block(fmt, block, out);
+    return QMOE_OK;
+}
 
 extern "C" int qmoe_linear_cpu(const void* w, int fmt, int n, int k, const float* x, int tokens, float* y) {
     if (!w || !x || !y) return fail(QMOE_EINVAL, "qmoe_linear_cpu: null pointer");

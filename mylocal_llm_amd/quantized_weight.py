@@ -3,11 +3,11 @@
 Mirrors ``PackedGGUFWeight`` of the reference (mini_llm/ops/quantized_weight.py:44-99):
 validation of shape / block alignment / byte count, a flat uint8 *view* of the caller's
 buffer (an mmap stays the owner), and zero-copy ``select_outer``.  Constructing it never
-materialises a floating-point matrix.  Decoding happens on the device only: the
-``*_reference`` methods of the reference's container (mini_llm/ops/quantized_weight.py:101-250,
-NumPy decoders there) keep their names, arguments and errors here but upload the packed rows
-they need and run the device decoder / linear; this package has no host decoder, and they
-raise without a HIP device.
+materialises a floating-point matrix.  The ``*_reference`` methods of the reference's container
+(mini_llm/ops/quantized_weight.py:101-250, NumPy decoders there) keep their names, arguments and
+errors and are host functions here too: they run the scalar C++ decoder / linear of the
+library's host twins (``qmoe_dequantize_cpu`` / ``qmoe_linear_cpu``), whose decoded values are
+those of the device decoder bit for bit.  None of them touches the GPU.
 """
 from dataclasses import dataclass
 import math
@@ -85,26 +85,32 @@ class PackedGGUFWeight:
         return PackedGGUFWeight(self.data[start * row_bytes:stop * row_bytes],
                                 (stop - start, self.shape[1]), self.quant_type)
 
-    # ---- the reference's host helpers, computed on the device --------------------------------
+    # ---- the reference's host helpers, on the library's host twins -----------------------------
     @staticmethod
     def _reference_tile_rows(tile_rows):
         if isinstance(tile_rows, (bool, np.bool_)) or not isinstance(tile_rows, (int, np.integer)) or tile_rows <= 0:
             raise ValueError("tile_rows must be a positive integer")
         return int(tile_rows)
 
-    def _device_matrix(self, data, rows):
-        from .quantized_linear import packed_to_device
-        return packed_to_device(PackedGGUFWeight(data, (rows, self.shape[-1]), self.quant_type))
+    def _decode_rows(self, raw, rows):
+        """fp32 [rows, columns] of ``rows`` packed rows lying contiguously in ``raw``."""
+        import ctypes
+        from . import _lib
+        raw = np.ascontiguousarray(np.asarray(raw).reshape(-1).view(np.uint8))
+        out = np.empty((rows, self.shape[-1]), dtype=np.float32)
+        if rows:
+            rc = _lib.load().qmoe_dequantize_cpu(ctypes.c_void_p(raw.ctypes.data), _lib.FORMAT_ID[self.quant_type], rows,
+                                                 self.shape[-1], ctypes.c_void_p(out.ctypes.data))
+            _lib.check(rc, "Host dequantize")
+        return out
 
     def dequantize_reference(self):
-        """fp32 ndarray of ``shape``, bit-identical to quantized_weight.py:151-250 (device decoder)."""
-        rows = math.prod(self.shape[:-1])
-        dense = self._device_matrix(self.data, rows).dequantize()
-        return dense.cpu().numpy().reshape(self.shape)
+        """fp32 ndarray of ``shape``, bit-identical to quantized_weight.py:151-250."""
+        return self._decode_rows(self.data, math.prod(self.shape[:-1])).reshape(self.shape)
 
     def dequantize_rows_reference(self, indices, *, tile_rows=32):
         """Selected rows of a matrix, order and duplicates preserved (quantized_weight.py:101-125);
-        only the requested rows are uploaded and decoded, ``tile_rows`` of them at a time."""
+        only the requested rows are decoded, ``tile_rows`` of them at a time."""
         if len(self.shape) != 2:
             raise ValueError("selected rows require a matrix; select_outer first")
         tile_rows = self._reference_tile_rows(tile_rows)
@@ -117,28 +123,17 @@ class PackedGGUFWeight:
         raw = self.data.reshape(self.shape[0], self.nbytes // self.shape[0])
         for start in range(0, len(indices), tile_rows):
             selected = indices[start:start + tile_rows]
-            tile = self._device_matrix(np.ascontiguousarray(raw[selected]), len(selected))
-            result[start:start + len(selected)] = tile.dequantize().cpu().numpy()
+            result[start:start + len(selected)] = self._decode_rows(raw[selected], len(selected))
         return result
 
     def matvec_reference(self, vector, *, tile_rows=32):
-        """fp32 ``W @ vector`` (quantized_weight.py:133-149): packed rows go to the device
-        ``tile_rows`` at a time and through the single-token linear."""
+        """fp32 ``W @ vector`` (quantized_weight.py:133-149) through the host linear; ``tile_rows`` is
+        validated as in the reference (the host linear walks row by row and needs no tiling)."""
         if len(self.shape) != 2:
             raise ValueError("matvec requires a matrix; select_outer first")
-        tile_rows = self._reference_tile_rows(tile_rows)
+        self._reference_tile_rows(tile_rows)
         vector = np.asarray(vector, dtype=np.float32)
         if vector.shape != (self.shape[1],):
             raise ValueError("vector shape must equal (matrix columns,)")
-        import torch
-        from .quantized_linear import quantized_linear
-        result = np.empty(self.shape[0], dtype=np.float32)
-        row_bytes = self.nbytes // self.shape[0]
-        x = None
-        for start in range(0, self.shape[0], tile_rows):
-            end = min(start + tile_rows, self.shape[0])
-            tile = self._device_matrix(self.data[start * row_bytes:end * row_bytes], end - start)
-            if x is None:
-                x = torch.from_numpy(np.ascontiguousarray(vector)[None]).to(tile.data.device)
-            result[start:end] = quantized_linear(x, tile).cpu().numpy()[0]
-        return result
+        from .native_packed_cpu import packed_cpu_linear
+        return packed_cpu_linear(vector[None], self)[0]

@@ -94,32 +94,3 @@ def test_full_size_matrix_bit_exact(cuda, fmt, shape):
     w = synthetic.packed_weight(fmt, shape, 106)
     got = upload(w, cuda).dequantize().cpu().numpy()
     np.testing.assert_array_equal(bits(got), bits(R.dequantize(w.data, shape, fmt)))
-
-
-@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_K", "Q5_K", "Q6_K", "BF16"])
-def test_container_reference_helpers_run_on_the_device(cuda, fmt):
-    """PackedGGUFWeight.dequantize_reference / dequantize_rows_reference / matvec_reference keep the
-    reference's names, arguments and errors (quantized_weight.py:101-250); the arithmetic is the
-    device decoder's and matches the oracle bit for bit (matvec: to fp32 rounding)."""
-    w = synthetic.packed_weight(fmt, (3, 40, 512), 77)
-    dense = R.dequantize(w.data, w.shape, fmt)
-    np.testing.assert_array_equal(w.dequantize_reference().view(np.uint32), dense.view(np.uint32))
-    one = w.select_outer(1)
-    idx = np.array([39, 0, 7, 7, 12], np.int64)
-    rows = one.dequantize_rows_reference(idx, tile_rows=2)
-    np.testing.assert_array_equal(rows.view(np.uint32), dense[1][idx].view(np.uint32))
-    x = synthetic.activations((512,), 78)
-    y = one.matvec_reference(x, tile_rows=16)
-    want = R.linear(x[None], one.data, one.shape, fmt)[0]
-    assert y.shape == (40,) and y.dtype == np.float32
-    assert np.linalg.norm(y - want) <= 2e-6 * np.linalg.norm(want)
-    with pytest.raises(ValueError, match="matrix"):
-        w.matvec_reference(x)
-    with pytest.raises(ValueError, match="tile_rows"):
-        one.matvec_reference(x, tile_rows=0)
-    with pytest.raises(ValueError, match="vector shape"):
-        one.matvec_reference(x[:-1])
-    with pytest.raises(IndexError):
-        one.dequantize_rows_reference(np.array([40]))
-    with pytest.raises(ValueError, match="integer"):
-        one.dequantize_rows_reference(np.array([0.5]))

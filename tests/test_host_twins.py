@@ -89,6 +89,36 @@ def test_decoded_weights_are_those_of_the_reference_decoder(fmt):
     np.testing.assert_array_equal(quantized_linear(np.eye(k, dtype=np.float32), w).T, dense)
 
 
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q4_0", "Q4_K", "Q3_K", "Q5_K", "Q6_K", "BF16"])
+def test_container_reference_helpers_are_host_functions(fmt):
+    """PackedGGUFWeight.dequantize_reference / dequantize_rows_reference / matvec_reference keep the
+    reference's names, arguments and errors (quantized_weight.py:101-250); the arithmetic is the
+    library's host decoder and matches the oracle bit for bit (matvec: to fp32 rounding)."""
+    w = synthetic.packed_weight(fmt, (3, 40, 512), 77)
+    dense = R.dequantize(w.data, w.shape, fmt)
+    np.testing.assert_array_equal(w.dequantize_reference().view(np.uint32), dense.view(np.uint32))
+    one = w.select_outer(1)
+    idx = np.array([39, 0, 7, 7, 12], np.int64)
+    rows = one.dequantize_rows_reference(idx, tile_rows=2)
+    np.testing.assert_array_equal(rows.view(np.uint32), dense[1][idx].view(np.uint32))
+    x = synthetic.activations((512,), 78)
+    y = one.matvec_reference(x, tile_rows=16)
+    want = R.linear(x[None], one.data, one.shape, fmt)[0]
+    assert y.shape == (40,) and y.dtype == np.float32
+    assert np.linalg.norm(y - want) <= 2e-6 * np.linalg.norm(want)
+    with pytest.raises(ValueError, match="matrix"):
+        w.matvec_reference(x)
+    with pytest.raises(ValueError, match="tile_rows"):
+        one.matvec_reference(x, tile_rows=0)
+    with pytest.raises(ValueError, match="vector shape"):
+        one.matvec_reference(x[:-1])
+    with pytest.raises(IndexError):
+        one.dequantize_rows_reference(np.array([40]))
+    with pytest.raises(ValueError, match="integer"):
+        one.dequantize_rows_reference(np.array([0.5]))
+
+
+
 def test_swiglu_mixed_formats_and_shapes():
     gate = synthetic.packed_weight("Q4_K", (48, 512), 3)
     up = synthetic.packed_weight("Q6_K", (48, 512), 4)
