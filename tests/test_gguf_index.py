@@ -227,3 +227,60 @@ def test_index_over_a_written_file_and_spec(tmp_path, fused):
     idx.reader.fields["qwen3next.expert_group_count"] = Field(2)
     with pytest.raises(NotImplementedError, match="expert_group_count"):
         Qwen3NextMoESpec.from_index(idx, 0)
+
+
+# ---- single rows of an embedding-like tensor (the reference's tests/test_0106p_gguf_rows.py) ------
+def _row_tensor(kind):
+    from types import SimpleNamespace
+    values = (np.arange(5 * 32).reshape(5, 32) % 17 - 8).astype(np.float32) / 16
+    if kind == "Q8_0":
+        codes = (values * 16).astype(np.int8)
+        scale = np.full((5, 1), 1 / 16, dtype="<f2")
+        data = np.concatenate((scale.view(np.uint8), codes.view(np.uint8)), axis=1)
+    elif kind == "BF16":
+        data = (values.view(np.uint32) >> 16).astype("<u2").view(np.uint8)
+    else:
+        data = values.astype(np.float16 if kind == "F16" else np.float32)
+    return SimpleNamespace(name="embedding", shape=(32, 5), data=data, tensor_type=SimpleNamespace(name=kind)), values
+
+
+@pytest.mark.parametrize("kind", ["F32", "F16", "BF16", "Q8_0"])
+def test_single_rows_decode_only_the_row_and_leave_the_owner_alone(kind, monkeypatch):
+    from mylocal_llm_amd.gguf_tensor import decode_gguf_row
+    weight, expected = _row_tensor(kind)
+    before, writable = weight.data.copy(), weight.data.flags.writeable
+    decoded_shapes = []
+    whole = PackedGGUFWeight.dequantize_reference
+
+    def only_rows(self):
+        decoded_shapes.append(self.shape)
+        assert self.shape == (32,), "the whole table must never be expanded"
+        return whole(self)
+
+    monkeypatch.setattr(PackedGGUFWeight, "dequantize_reference", only_rows)
+    for row in (4, 0, 2):
+        np.testing.assert_array_equal(decode_gguf_row(weight, row), expected[row])
+    assert len(decoded_shapes) == (3 if kind == "Q8_0" else 0)
+    np.testing.assert_array_equal(weight.data, before)
+    assert weight.data.flags.writeable == writable
+
+
+@pytest.mark.parametrize("row,error", [(-1, IndexError), (5, IndexError), (True, TypeError), (1.0, TypeError)])
+def test_single_row_index_is_validated(row, error):
+    from mylocal_llm_amd.gguf_tensor import decode_gguf_row
+    with pytest.raises(error):
+        decode_gguf_row(_row_tensor("Q8_0")[0], row)
+
+
+def test_single_row_of_big_endian_bf16_words_and_a_short_payload():
+    from mylocal_llm_amd.gguf_tensor import decode_gguf_row
+    weight, expected = _row_tensor("BF16")
+    weight.data = weight.data.view("<u2").astype(">u2")
+    np.testing.assert_array_equal(decode_gguf_row(weight, 3), expected[3])
+    weight.data = weight.data[:-1]
+    with pytest.raises(ValueError, match="payload"):
+        decode_gguf_row(weight, 0)
+    weight3 = _row_tensor("F32")[0]
+    weight3.shape = (32, 5, 1)
+    with pytest.raises(ValueError, match="positive matrix"):
+        decode_gguf_row(weight3, 0)
