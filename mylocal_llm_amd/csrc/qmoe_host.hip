@@ -16,6 +16,10 @@
 #include "qmoe_common.hpp"
 #include "qmoe_formats.hpp"
 
+// The decoders round a product before they subtract from it, as the reference does: a fused
+// multiply-add would change the last bit of a weight.
+#pragma clang fp contract(off)
+
 namespace {
 
 using qmoe::block_bytes;
