@@ -6,7 +6,6 @@ widened to fp32 with integer shifts only, so signed zeros and every NaN payload 
 (quantised) tensors never pass through here.
 """
 from numbers import Integral
-from types import SimpleNamespace
 
 import numpy as np
 
@@ -57,39 +56,48 @@ def decode_gguf_dense(tensor):
     return decoder(tensor, canonical_shape(tensor))
 
 
-def _bf16_row_payload(tensor, shape, row):
-    """The bytes (or words) of one row of a BF16 matrix, still undecoded."""
+def _row_of_typed(tensor, shape, row):
+    return _typed_view(tensor, shape)[row]
+
+
+def _row_of_bf16(tensor, shape, row):
+    """Row ``row`` of a BF16 matrix: its 2 * width bytes (or width words) are cut out of the payload
+    first and only they are widened."""
     payload = np.asarray(tensor.data)
-    rows, width = shape
-    if not payload.flags.c_contiguous or payload.nbytes != 2 * rows * width:
+    width = shape[1]
+    if payload.nbytes != 2 * shape[0] * width or not payload.flags.c_contiguous:
         raise ValueError(f"{tensor.name}: invalid contiguous BF16 matrix payload")
-    if payload.dtype == np.uint8:
-        flat = payload.reshape(-1)
-        return flat[2 * width * row:2 * width * (row + 1)]
-    if payload.dtype.kind == "u" and payload.dtype.itemsize == 2:
-        return payload.reshape(shape)[row]
-    raise ValueError(f"{tensor.name}: BF16 row payload must be uint8 or uint16")
+    per_row = {1: 2 * width, 2: width}.get(payload.dtype.itemsize if payload.dtype.kind == "u" else 0)
+    if per_row is None:
+        raise ValueError(f"{tensor.name}: BF16 row payload must be uint8 or uint16")
+    cut = payload.reshape(-1)[per_row * row:per_row * (row + 1)]
+    wide = _bf16_words(tensor, cut).astype(np.uint32)
+    wide <<= 16
+    return wide.view(np.float32)
+
+
+def _row_of_packed(tensor, shape, row):
+    from .quantized_weight import PackedGGUFWeight
+    return PackedGGUFWeight(tensor.data, shape, tensor.tensor_type.name).select_outer(row).dequantize_reference()
+
+
+_ROW_READERS = {"F32": _row_of_typed, "F16": _row_of_typed, "BF16": _row_of_bf16}
 
 
 def decode_gguf_row(tensor, row):
     """One row of a canonical [rows, width] tensor without expanding the rest of it
     (mini_llm/external/gguf_tensor.py:54-89): a packed tensor decodes the blocks of that row only,
     BF16 is sliced as bytes before it is widened, F32 / F16 rows are views of the reader's array."""
-    from .quantized_weight import BLOCK_FORMATS, PackedGGUFWeight
+    from .quantized_weight import BLOCK_FORMATS
     shape = canonical_shape(tensor)
     if len(shape) != 2 or min(shape) <= 0:
         raise ValueError(f"{tensor.name}: row access requires a positive matrix shape")
     if isinstance(row, bool) or not isinstance(row, Integral):
         raise TypeError("row must be an integer")
-    if row < 0 or row >= shape[0]:
+    if row not in range(shape[0]):
         raise IndexError(row)
     kind = tensor.tensor_type.name
-    if kind == "BF16":
-        one = SimpleNamespace(name=tensor.name, shape=(shape[1],), tensor_type=tensor.tensor_type,
-                              data=_bf16_row_payload(tensor, shape, int(row)))
-        return decode_gguf_dense(one)
-    if kind in BLOCK_FORMATS:
-        return PackedGGUFWeight(tensor.data, shape, kind).select_outer(int(row)).dequantize_reference()
-    if kind in DENSE_KINDS:
-        return decode_gguf_dense(tensor)[row]
-    raise NotImplementedError(f"{tensor.name}: unsupported row type {kind}")
+    reader = _ROW_READERS.get(kind) or (_row_of_packed if kind in BLOCK_FORMATS else None)
+    if reader is None:
+        raise NotImplementedError(f"{tensor.name}: unsupported row type {kind}")
+    return reader(tensor, shape, int(row))

@@ -19,49 +19,69 @@ from .quantized_linear import (
 from .quantized_weight import BLOCK_FORMATS
 
 
+def _is_index(value, bound):
+    return isinstance(value, (int, np.integer)) and not isinstance(value, bool) and 0 <= value < bound
+
+
+def _device_f32(t):
+    return isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32
+
+
+def _storage_ok(w):
+    """The packed bytes of one projection are a contiguous uint8 tensor of exactly the size its shape asks for."""
+    per_block, block_size = BLOCK_FORMATS[w.quant_type]
+    rows, cols = w.shape
+    return (w.data.dtype == torch.uint8 and w.data.is_contiguous() and cols % per_block == 0
+            and w.data.numel() == rows * cols // per_block * block_size)
+
+
+def _operand_checks(x, experts, routes, block_k, slots):
+    """(passes, reason) pairs about the call's own operands, cheapest first; evaluated lazily."""
+    yield block_k in (256, 512, 1024), "block_k must be 256, 512 or 1024"
+    yield _device_f32(x), "x must be a CUDA FP32 tensor"
+    yield (x.ndim == 2 and x.shape[0] == 1 and x.shape[1] > 0 and x.is_contiguous()), \
+        "x must be contiguous [1, D] with positive D"
+    yield (isinstance(experts, (list, tuple)) and 0 < len(experts) < 65536), \
+        "experts must be a nonempty list/tuple of at most 65535 handles"
+    count = len(experts)
+    if slots is not None:
+        yield (isinstance(slots, (tuple, list)) and len(slots) == count and all(_is_index(s, count) for s in slots)), \
+            "routing_slots must be host integer indices into the [E] routing weights"
+    yield (_device_f32(routes) and tuple(routes.shape) == (count,)), \
+        "routing_weights must be a CUDA FP32 [E] tensor (slices allowed)"
+    yield routes.device == x.device, "all operands must be on the same device"
+
+
+def _handle_checks(x, handle, first):
+    """(passes, reason) pairs about one expert handle; ``first`` is the handle all others must match."""
+    yield isinstance(handle, PackedExpertFFNInference), "experts must contain PackedExpertFFNInference handles"
+    triple = (handle.gate, handle.up, handle.down)
+    yield all(isinstance(w, DevicePackedGGUFWeight) for w in triple), \
+        "all projections must be DevicePackedGGUFWeight (no host fallback)"
+    d = x.shape[1]
+    gate_shape = tuple(handle.gate.shape)
+    yield (len(gate_shape) == 2 and min(gate_shape) > 0 and gate_shape[1] == d
+           and tuple(handle.up.shape) == gate_shape and tuple(handle.down.shape) == gate_shape[::-1]), \
+        "expert shapes must be gate/up [F, D], down [D, F] matching x"
+    if handle is not first:
+        same = all((tuple(w.shape), w.quant_type) == (tuple(v.shape), v.quant_type)
+                   for w, v in zip(triple, (first.gate, first.up, first.down)))
+        yield same, "all experts must share per-projection shapes and quantization formats"
+    for w in triple:
+        yield _storage_ok(w), "invalid packed projection storage or block alignment"
+        yield w.data.device == x.device, "all operands must be on the same device"
+
+
 def _unsupported_reason(x, experts, routing_weights, block_k, routing_slots=None):
-    if block_k not in (256, 512, 1024):
-        return "block_k must be 256, 512 or 1024"
-    if not isinstance(x, torch.Tensor) or not x.is_cuda or x.dtype != torch.float32:
-        return "x must be a CUDA FP32 tensor"
-    if x.ndim != 2 or x.shape[0] != 1 or x.shape[1] <= 0 or not x.is_contiguous():
-        return "x must be contiguous [1, D] with positive D"
-    if not isinstance(experts, (list, tuple)) or not 1 <= len(experts) <= 65535:
-        return "experts must be a nonempty list/tuple of at most 65535 handles"
-    if routing_slots is not None and (
-            not isinstance(routing_slots, (tuple, list)) or len(routing_slots) != len(experts)
-            or any(not isinstance(slot, (int, np.integer)) or isinstance(slot, bool)
-                   or not 0 <= slot < len(experts) for slot in routing_slots)):
-        return "routing_slots must be host integer indices into the [E] routing weights"
-    if (not isinstance(routing_weights, torch.Tensor) or not routing_weights.is_cuda
-            or routing_weights.dtype != torch.float32
-            or tuple(routing_weights.shape) != (len(experts),)):
-        return "routing_weights must be a CUDA FP32 [E] tensor (slices allowed)"
-    if routing_weights.device != x.device:
-        return "all operands must be on the same device"
-    signature = None
-    for expert in experts:
-        if not isinstance(expert, PackedExpertFFNInference):
-            return "experts must contain PackedExpertFFNInference handles"
-        projections = (expert.gate, expert.up, expert.down)
-        if not all(isinstance(w, DevicePackedGGUFWeight) for w in projections):
-            return "all projections must be DevicePackedGGUFWeight (no host fallback)"
-        gate, up, down = projections
-        if (len(gate.shape) != 2 or min(gate.shape) <= 0
-                or gate.shape != up.shape or gate.shape[1] != x.shape[1]
-                or down.shape != (x.shape[1], gate.shape[0])):
-            return "expert shapes must be gate/up [F, D], down [D, F] matching x"
-        current = tuple((w.shape, w.quant_type) for w in projections)
-        if signature is not None and current != signature:
-            return "all experts must share per-projection shapes and quantization formats"
-        signature = current
-        for w in projections:
-            qk, qb = BLOCK_FORMATS[w.quant_type]
-            if (w.data.dtype != torch.uint8 or not w.data.is_contiguous() or w.shape[1] % qk
-                    or w.data.numel() != w.shape[0] * w.shape[1] // qk * qb):
-                return "invalid packed projection storage or block alignment"
-            if w.data.device != x.device:
-                return "all operands must be on the same device"
+    """None if the call is one the grouped path takes, else the reason (the conditions of
+    mini_llm/ops/grouped_quantized_experts.py:82-138 that apply to device tensors)."""
+    for passes, reason in _operand_checks(x, experts, routing_weights, block_k, routing_slots):
+        if not passes:
+            return reason
+    for handle in experts:
+        for passes, reason in _handle_checks(x, handle, experts[0]):
+            if not passes:
+                return reason
     return None
 
 

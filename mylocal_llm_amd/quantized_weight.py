@@ -9,8 +9,10 @@ errors and are host functions here too: they run the scalar C++ decoder / linear
 library's host twins (``qmoe_dequantize_cpu`` / ``qmoe_linear_cpu``), whose decoded values are
 those of the device decoder bit for bit.  None of them touches the GPU.
 """
+import ctypes
+import operator
 from dataclasses import dataclass
-import math
+from functools import reduce
 
 import numpy as np
 
@@ -29,6 +31,24 @@ BLOCK_FORMATS = {
 }
 
 
+def _count(dims):
+    return reduce(operator.mul, dims, 1)
+
+
+def _packed_bytes(quant_type, dims):
+    """Bytes that ``dims`` elements take in ``quant_type`` (the innermost dimension is whole blocks)."""
+    per_block, block_size = BLOCK_FORMATS[quant_type]
+    return _count(dims) // per_block * block_size
+
+
+def _positive_int(value, message):
+    """``value`` as an int if it is a true integer above zero (a bool is not), else ValueError."""
+    is_integer = isinstance(value, (int, np.integer)) and not isinstance(value, (bool, np.bool_))
+    if not is_integer or value <= 0:
+        raise ValueError(message)
+    return int(value)
+
+
 @dataclass(frozen=True)
 class PackedGGUFWeight:
     """Validated packed tensor in canonical row-major shape; ``data`` aliases the owner."""
@@ -38,23 +58,24 @@ class PackedGGUFWeight:
     quant_type: str
 
     def __post_init__(self):
-        if self.quant_type not in BLOCK_FORMATS:
-            raise ValueError(f"Unsupported packed GGUF type: {self.quant_type}")
-        shape = tuple(int(d) for d in self.shape)
-        if not shape or any(d <= 0 for d in shape):
+        fmt = self.quant_type
+        geometry = BLOCK_FORMATS.get(fmt)
+        if geometry is None:
+            raise ValueError(f"Unsupported packed GGUF type: {fmt}")
+        dims = tuple(map(int, self.shape))
+        if len(dims) == 0 or min(dims) <= 0:
             raise ValueError("Packed GGUF shape must have positive dimensions")
-        elems, nbytes = BLOCK_FORMATS[self.quant_type]
-        if shape[-1] % elems:
-            raise ValueError(f"GGUF {self.quant_type}: innermost dimension must be a multiple of {elems}")
-        raw = np.asarray(self.data)
-        if not raw.flags.c_contiguous:
+        if dims[-1] % geometry[0] != 0:
+            raise ValueError(f"GGUF {fmt}: innermost dimension must be a multiple of {geometry[0]}")
+        payload = np.asarray(self.data)
+        if not payload.flags.c_contiguous:
             raise ValueError("GGUF packed data must be contiguous")
-        raw = raw.view(np.uint8).reshape(-1)
-        expected = math.prod(shape) // elems * nbytes
-        if raw.size != expected:
-            raise ValueError(f"GGUF {self.quant_type}: expected {expected} bytes, got {raw.size}")
-        object.__setattr__(self, "shape", shape)
-        object.__setattr__(self, "data", raw)
+        flat = payload.view(np.uint8).reshape(-1)   # a view: the caller's buffer (an mmap) stays the owner
+        want = _packed_bytes(fmt, dims)
+        if flat.size != want:
+            raise ValueError(f"GGUF {fmt}: expected {want} bytes, got {flat.size}")
+        for name, value in (("shape", dims), ("data", flat)):
+            object.__setattr__(self, name, value)
 
     @property
     def nbytes(self):
@@ -64,16 +85,24 @@ class PackedGGUFWeight:
     def block_elements(self):
         return BLOCK_FORMATS[self.quant_type][0]
 
+    @property
+    def _row_bytes(self):
+        return _packed_bytes(self.quant_type, self.shape[-1:])
+
+    def _view(self, first_byte, dims):
+        """Zero-copy sub-tensor of shape ``dims`` that starts ``first_byte`` bytes into the payload."""
+        size = _packed_bytes(self.quant_type, dims)
+        return PackedGGUFWeight(self.data[first_byte:first_byte + size], tuple(dims), self.quant_type)
+
     def select_outer(self, index):
         """Zero-copy slice along the leading dimension (one expert of [E, N, K])."""
         if len(self.shape) < 2:
             raise ValueError("select_outer requires at least two dimensions")
-        if not 0 <= int(index) < self.shape[0]:
+        which = int(index)
+        if which < 0 or which >= self.shape[0]:
             raise IndexError(index)
-        elems, nbytes = BLOCK_FORMATS[self.quant_type]
-        chunk = math.prod(self.shape[1:]) // elems * nbytes
-        begin = int(index) * chunk
-        return PackedGGUFWeight(self.data[begin:begin + chunk], self.shape[1:], self.quant_type)
+        inner = self.shape[1:]
+        return self._view(which * _packed_bytes(self.quant_type, inner), inner)
 
     def select_rows(self, start, stop):
         """Zero-copy row range of a matrix (e.g. the gate or up half of a fused gate_up)."""
@@ -81,20 +110,15 @@ class PackedGGUFWeight:
             raise ValueError("select_rows requires a matrix; select_outer first")
         if not 0 <= start < stop <= self.shape[0]:
             raise IndexError((start, stop))
-        row_bytes = self.nbytes // self.shape[0]
-        return PackedGGUFWeight(self.data[start * row_bytes:stop * row_bytes],
-                                (stop - start, self.shape[1]), self.quant_type)
+        return self._view(start * self._row_bytes, (stop - start, self.shape[1]))
 
     # ---- the reference's host helpers, on the library's host twins -----------------------------
     @staticmethod
     def _reference_tile_rows(tile_rows):
-        if isinstance(tile_rows, (bool, np.bool_)) or not isinstance(tile_rows, (int, np.integer)) or tile_rows <= 0:
-            raise ValueError("tile_rows must be a positive integer")
-        return int(tile_rows)
+        return _positive_int(tile_rows, "tile_rows must be a positive integer")
 
     def _decode_rows(self, raw, rows):
         """fp32 [rows, columns] of ``rows`` packed rows lying contiguously in ``raw``."""
-        import ctypes
         from . import _lib
         raw = np.ascontiguousarray(np.asarray(raw).reshape(-1).view(np.uint8))
         out = np.empty((rows, self.shape[-1]), dtype=np.float32)
@@ -106,25 +130,26 @@ class PackedGGUFWeight:
 
     def dequantize_reference(self):
         """fp32 ndarray of ``shape``, bit-identical to quantized_weight.py:151-250."""
-        return self._decode_rows(self.data, math.prod(self.shape[:-1])).reshape(self.shape)
+        return self._decode_rows(self.data, _count(self.shape[:-1])).reshape(self.shape)
 
     def dequantize_rows_reference(self, indices, *, tile_rows=32):
         """Selected rows of a matrix, order and duplicates preserved (quantized_weight.py:101-125);
         only the requested rows are decoded, ``tile_rows`` of them at a time."""
         if len(self.shape) != 2:
             raise ValueError("selected rows require a matrix; select_outer first")
-        tile_rows = self._reference_tile_rows(tile_rows)
-        indices = np.asarray(indices)
-        if indices.ndim != 1 or indices.dtype.kind not in "iu":
+        step = self._reference_tile_rows(tile_rows)
+        wanted = np.asarray(indices)
+        if wanted.ndim != 1 or wanted.dtype.kind not in "iu":
             raise ValueError("indices must be a one-dimensional integer array")
-        if np.any(indices >= self.shape[0]) or np.any(indices < 0):
+        n_rows, n_cols = self.shape
+        if wanted.size and (int(wanted.min()) < 0 or int(wanted.max()) >= n_rows):
             raise IndexError("packed row index out of range")
-        result = np.empty((len(indices), self.shape[1]), dtype=np.float32)
-        raw = self.data.reshape(self.shape[0], self.nbytes // self.shape[0])
-        for start in range(0, len(indices), tile_rows):
-            selected = indices[start:start + tile_rows]
-            result[start:start + len(selected)] = self._decode_rows(raw[selected], len(selected))
-        return result
+        by_row = self.data.reshape(n_rows, self._row_bytes)
+        pieces = [self._decode_rows(by_row[wanted[at:at + step]], len(wanted[at:at + step]))
+                  for at in range(0, wanted.size, step)]
+        if not pieces:
+            return np.empty((0, n_cols), dtype=np.float32)
+        return np.concatenate(pieces, axis=0)
 
     def matvec_reference(self, vector, *, tile_rows=32):
         """fp32 ``W @ vector`` (quantized_weight.py:133-149) through the host linear; ``tile_rows`` is
