@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define QMOE_ABI_VERSION 3
+#define QMOE_ABI_VERSION 4
 
 /* Packed formats.  Ids 0..5 are the reference's (_FORMAT_ID,
  * mini_llm/ops/quantized_linear.py:34 and native_packed_cpu.cpp:12).  BF16 has no
@@ -59,6 +59,27 @@ enum {
 
 int qmoe_abi_version(void);
 const char* qmoe_last_error(void);
+
+/* Optional set-up of the current device ahead of the first compute call: resolves the addresses
+ * of the library's per-GPU device variables (the launch status word and the scratch array of
+ * qmoe_moe_forward_static), which the compute calls otherwise do on their first use on a device.
+ * Call it once per device before recording a HIP graph: looking a device variable up is not
+ * stream work and is not allowed while a stream captures.  No counterpart in the reference. */
+int qmoe_init(void);
+
+/* Waits inside the streaming kernels (a wave waiting for the other waves of its own workgroup)
+ * are bounded in wall-clock time.  A wave whose wait expires raises the current device's launch
+ * status word, stores no further results and runs to its end, so the launch ends normally and its
+ * outputs are incomplete rather than wrong.  qmoe_check_status SYNCHRONISES `stream`, reads the
+ * word and clears it: QMOE_OK if no launch on this device gave up since the last check, else
+ * QMOE_ELAUNCH (the only call of this library that waits for the device).  No counterpart in
+ * the reference, whose kernels have no waits. */
+int qmoe_check_status(void* stream);
+
+/* The bound of those waits in ticks of the 100 MHz device counter; 0 restores the default (one
+ * second).  A negative value makes every wait expire at once: the host-forced way to exercise
+ * the give-up path, every kernel still ends normally. */
+void qmoe_set_wait_limit(long long ticks);
 
 /* Elements and bytes per block of a format (BLOCK_FORMATS,
  * mini_llm/ops/quantized_weight.py:24-37). */

@@ -6,7 +6,7 @@ from concurrent.futures import ThreadPoolExecutor
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libqmoe_hip.so")
-SOURCES = ("qmoe_linear.hip", "qmoe_stream.hip", "qmoe_span.hip", "qmoe_router.hip", "qmoe_moe.hip", "qmoe_decode.hip", "qmoe_gemm.hip", "qmoe_front.hip", "qmoe_few.hip", "qmoe_host.hip", "qmoe_probe.hip")
+SOURCES = ("qmoe_linear.hip", "qmoe_stream.hip", "qmoe_span.hip", "qmoe_router.hip", "qmoe_moe.hip", "qmoe_decode.hip", "qmoe_gemm.hip", "qmoe_front.hip", "qmoe_few.hip", "qmoe_host.hip", "qmoe_probe.hip", "qmoe_status.hip")
 # Packed fp32 VALU forms are switched off for all device code.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -43,11 +43,14 @@ class MoeArgs(ctypes.Structure):
                 ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P), ("status_out", _P)]
 
 
-ABI_VERSION = 3   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
+ABI_VERSION = 4   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
 
 _SIGNATURES = {
     "qmoe_abi_version": ([], _I),
     "qmoe_last_error": ([], ctypes.c_char_p),
+    "qmoe_init": ([], _I),
+    "qmoe_check_status": ([_P], _I),
+    "qmoe_set_wait_limit": ([ctypes.c_longlong], None),
     "qmoe_format_info": ([_I, ctypes.POINTER(_I), ctypes.POINTER(_I)], _I),
     "qmoe_dequantize": ([_P, _I, _I64, _I64, _P, _P], _I),
     "qmoe_linear": ([_P, _I, _I, _I, _P, _I, _I, _P, _I, _P], _I),

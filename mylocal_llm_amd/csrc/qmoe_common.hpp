@@ -15,6 +15,16 @@ char* error_buffer();
 int fail(int status, const char* fmt, ...);
 int check_launch(const char* what);
 
+// ---- launch status ---------------------------------------------------------------------------
+// One word per GPU inside the library's device image.  Kernels with bounded waits raise bits in
+// it (vector stores) instead of hanging or returning wrong results silently; qmoe_check_status
+// reads and clears it.  launch_status_word gives the word's address on the current device
+// (resolved once per device), wait_limit_ticks the bound of such a wait in 100 MHz ticks.
+static constexpr uint32_t QMOE_STATUS_WAIT_EXPIRED = 1u;
+int launch_status_word(uint32_t** out);
+int64_t wait_limit_ticks();
+int static_scratch(void** out);
+
 // ---- global memory access ----------------------------------------------------------------
 // Pointers that reach a kernel inside an argument struct or through LDS carry no address
 // space, and loads through them become FLAT instructions: those may complete out of order, so

@@ -688,7 +688,8 @@ int qmoe_moe_forward(const qmoe_moe_args* args, void* workspace, size_t workspac
 static constexpr size_t MOE_STATIC_SCRATCH_BYTES = QMOE_MOE_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[MOE_STATIC_SCRATCH_BYTES];
 
-static int static_scratch(void** out) {
+}  // extern "C"
+int qmoe::static_scratch(void** out) {
     static constexpr int MAX_DEVICES = 64;
     static std::mutex lock;
     static void* per_device[MAX_DEVICES] = {};
@@ -706,6 +707,7 @@ static int static_scratch(void** out) {
     *out = per_device[dev];
     return QMOE_OK;
 }
+extern "C" {
 
 size_t qmoe_moe_static_scratch_bytes(void) { return MOE_STATIC_SCRATCH_BYTES; }
 

@@ -232,9 +232,25 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
         wait_vmcnt<PD * SL::CHUNKS>();
         if (sig_keys && --sig_wait == 0) count_in();
     };
-    // (bounded: a wave that never sees the count gives up after a few milliseconds instead of hanging)
+    // A wait for the other waves of the workgroup is bounded in wall-clock time (args.wait_ticks of
+    // the 100 MHz counter; far longer than any launch streams).  A wave whose wait expires does not
+    // hang and does not pretend: it raises the launch's status word with a vector store, stores no
+    // more results, and runs on to its end so that every request it has made drains.  A negative
+    // limit makes every wait expire at once (a host-forced run of this branch).
+    bool failed = false;
     auto spin_until = [&](lds_counter counter) {
-        for (int spins = 0; spins < (1 << 18) && *(volatile QMOE_LDS uint32_t*)counter < SPAN_WAVES; ++spins) __builtin_amdgcn_s_sleep(1);
+        bool ok = args.wait_ticks >= 0 && *(volatile QMOE_LDS uint32_t*)counter >= SPAN_WAVES;
+        if (!ok && args.wait_ticks >= 0) {
+            const uint64_t t0 = wall_clock64();
+            do {
+                __builtin_amdgcn_s_sleep(1);
+                ok = *(volatile QMOE_LDS uint32_t*)counter >= SPAN_WAVES;
+            } while (!ok && (int64_t)(wall_clock64() - t0) <= args.wait_ticks);
+        }
+        if (!uniform((int)ok) && !failed) {
+            failed = true;
+            if (lane == 0) stg<uint32_t>(args.status, QMOE_STATUS_WAIT_EXPIRED);
+        }
     };
 
     // The first item of every wave is fixed (item `me`), so its request and the first activation
@@ -327,7 +343,7 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
                     v = silu_mul(v, up);
                 }
                 const int row = t * rpi + sub;
-                if (u == lr - 1 && row < n) store_out(y, ydt, row, v);
+                if (u == lr - 1 && row < n && !failed) store_out(y, ydt, row, v);
             }
         } else {
             // a wider row: its parts of 4096 columns one after the other, the lane's slice of the
@@ -353,7 +369,7 @@ __global__ __launch_bounds__(SPAN_THREADS, 1) void span_kernel(const SpanArgs ar
                     c_slot = c_slot + SLOT == RING ? 0 : c_slot + SLOT;
                 }
                 acc = group_sum<64>(acc);
-                if (lane == 63) store_out(y, ydt, t, acc);
+                if (lane == 63 && !failed) store_out(y, ydt, t, acc);
             }
         }
     }
@@ -408,6 +424,8 @@ static bool span_plan(const StreamArgs& in, SpanArgs* out) {
     }
     a.keys = key + 1;
     a.items = items;
+    a.status = nullptr;      // (the launcher fills in the device's status word and the wait limit)
+    a.wait_ticks = 0;
     if (out) *out = a;
     return true;
 }
@@ -427,9 +445,11 @@ static bool span_basic(const StreamArgs& args) {
 }
 
 template <int FMT, bool PAIR, int PD>
-static int span_launch_as(const SpanArgs& args, hipStream_t s) {
+static int span_launch_as(SpanArgs& args, hipStream_t s) {
     static bool configured = false;   // (benign if two threads both set it)
     constexpr int lds = SpanLayout<FMT, PD>::TOTAL;
+    if (int rc = launch_status_word(&args.status)) return rc;
+    args.wait_ticks = wait_limit_ticks();
     if (!configured) {
         if (hipFuncSetAttribute((const void*)span_kernel<FMT, PAIR, PD>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
             return fail(QMOE_ELAUNCH, "span kernel: cannot reserve %d bytes of LDS", lds);

@@ -141,6 +141,8 @@ struct SpanKey {
 };
 struct SpanArgs {
     int count, keys, items, pad;
+    uint32_t* status;     // the device's launch status word (a wave whose bounded wait expires raises it)
+    int64_t wait_ticks;   // bound of a wait for the workgroup's other waves, in 100 MHz ticks; < 0: expire at once
     SpanProblem p[STREAM_MAX_PROBLEMS];
     SpanKey key[SPAN_MAX_KEYS];
 };

@@ -355,10 +355,15 @@ def test_full_8b_layer_in_one_batch_single_token(cuda, fmt):
         got = outs[i].cpu().numpy()
         assert got.shape == (1, n)
         assert np.array_equal(got.view(np.uint32), again[i].cpu().numpy().view(np.uint32))
-        rows = np.unique(np.concatenate([[0, 1, n - 2, n - 1], rng.choice(n, 40, replace=False)]))
+        # whole stretches of rows across 64-row boundaries (the first and last 64 rows, 130 rows
+        # around three boundaries inside the matrix) plus scattered single rows
+        inner = [64 * int(b) for b in rng.choice(np.arange(2, n // 64 - 2), 3, replace=False)]
+        rows = np.unique(np.concatenate([np.arange(64), np.arange(n - 64, n), rng.choice(n, 40, replace=False)]
+                                        + [np.arange(b - 65, b + 65) for b in inner]))
         sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), fmt)
         want = R.linear(xs[groups[i]].cpu().numpy(), *triple(sub))
         assert rel_l2(got[:, rows], want) <= 2e-6, (i, n, k)
+        np.testing.assert_allclose(got[:, rows], want, rtol=0, atol=2e-5 * np.abs(want).max())
         assert np.isfinite(got).all()
 
 
@@ -414,3 +419,42 @@ def test_four_host_threads_on_their_own_streams_give_identical_bits(cuda):
     for t in threads:
         t.join()
     assert not failures, failures[:3]
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("tokens", [1, 16])
+def test_bf16_weights_at_the_8b_projection_shapes(cuda, shape, tokens):
+    """BF16 weights ~ N(0, 0.02) at every projection shape of the 8B layer, one token and sixteen:
+    stretches of rows (first, last, across a 64-row boundary) against the oracle for every token."""
+    announce("linear 8B shape BF16", shape, tokens)
+    n, k = shape
+    w = synthetic.packed_weight("BF16", (n, k), 506)
+    rng = np.random.default_rng(503)
+    x = rng.standard_normal((tokens, k), dtype=np.float32)
+    y = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    assert y.shape == (tokens, n) and np.isfinite(y).all()
+    mid = 64 * (n // 128)
+    rows = np.unique(np.concatenate([np.arange(40), np.arange(n - 40, n), np.arange(mid - 20, mid + 20), rng.choice(n, 24, replace=False)]))
+    sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), "BF16")
+    assert rel_l2(y[:, rows], R.linear(x, *triple(sub))) <= (2e-6 if tokens == 1 else 3e-5)
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K"])
+def test_output_projection_of_the_vocabulary_at_full_shape(cuda, fmt):
+    """The output projection of the reference's model at its real shape, 151 936 x 2048
+    (mini_llm/external/qwen3next_model.py:291-293), one token: 311 M weights through the
+    single-token streaming kernel; stretches of rows at the start, across the middle and up to the
+    very last row against the oracle, and every output finite."""
+    announce("linear vocabulary projection", fmt)
+    n, k = 151936, 2048
+    w = synthetic.packed_weight(fmt, (n, k), 606)
+    rng = np.random.default_rng(603)
+    x = rng.standard_normal((1, k), dtype=np.float32)
+    y = quantized_linear(torch.from_numpy(x).to(cuda), upload(w, cuda)).cpu().numpy()
+    assert y.shape == (1, n) and np.isfinite(y).all()
+    rows = np.unique(np.concatenate([np.arange(70), np.arange(n - 70, n), np.arange(n // 2 - 35, n // 2 + 35),
+                                     rng.choice(n, 200, replace=False)]))
+    sub = PackedGGUFWeight(w.data.reshape(n, -1)[rows].copy(), (len(rows), k), fmt)
+    want = R.linear(x, *triple(sub))
+    assert rel_l2(y[:, rows], want) <= 2e-6
+    np.testing.assert_allclose(y[:, rows], want, rtol=0, atol=2e-5 * np.abs(want).max())

@@ -272,34 +272,76 @@ def test_decode_config_512_experts_top10(cuda, fmt, tokens):
     assert not synthetic.has_topk_ties(logits, k)
     out, w, ids = moe_step(torch.from_numpy(hidden).to(cuda), bank, k, logits=torch.from_numpy(logits).to(cuda),
                            shared=dshared, shared_gate=torch.from_numpy(gate_vec).to(cuda), return_routing=True)
-    sample = sorted(set([0, tokens - 1]))
-    want, want_w, want_ids = oracle_step(hidden[sample], logits[sample], k, gate, up, down, shared, gate_vec)
-    np.testing.assert_array_equal(ids.cpu().numpy()[sample], want_ids)
-    np.testing.assert_allclose(w.cpu().numpy()[sample], want_w, rtol=2e-6, atol=2e-7)
-    assert rel_l2(out.cpu().numpy()[sample], want) <= 2e-5 <= REL_L2
+    # every token against the oracle (which decodes each selected expert once)
+    want, want_w, want_ids = oracle_step(hidden, logits, k, gate, up, down, shared, gate_vec)
+    np.testing.assert_array_equal(ids.cpu().numpy(), want_ids)
+    np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6, atol=2e-7)
+    got = out.cpu().numpy()
+    assert rel_l2(got, want) <= 2e-5 <= REL_L2
+    for t in range(tokens):
+        assert rel_l2(got[t], want[t]) <= 3e-5, t
 
 
-def test_prefill_config_512_tokens_zipf(cuda):
-    """Benchmark prefill configuration: T=512, Zipf(1.1) routing, Q8_0.  Size-independent
-    checks: every token's output equals the same token run alone (dispatch/compaction is
-    permutation-invariant), plus sampled tokens against the oracle."""
-    announce("moe prefill T=512")
+def prefill_sample(ids, e, want=32):
+    """Tokens that cover the corners of the token->expert plan: the first, a middle and the last
+    token of the busiest expert's list (its first, a middle and its last chunk of 32), the token
+    of an expert that only one token selected, tokens of the first and the last expert in use, then
+    evenly spaced ones up to ``want``."""
+    counts = np.bincount(ids.ravel(), minlength=e)
+    t = ids.shape[0]
+    picks = []
+    busiest = int(counts.argmax())
+    holders = np.nonzero((ids == busiest).any(axis=1))[0]
+    picks += [int(holders[0]), int(holders[len(holders) // 2]), int(holders[-1])]
+    if len(holders) > 33:
+        picks += [int(holders[31]), int(holders[32])]     # either side of a chunk boundary
+    singles = np.nonzero(counts == 1)[0]
+    if len(singles):
+        picks.append(int(np.nonzero((ids == singles[0]).any(axis=1))[0][0]))
+    used = np.nonzero(counts)[0]
+    for expert in (used[0], used[-1]):
+        picks.append(int(np.nonzero((ids == expert).any(axis=1))[0][-1]))
+    picks += [0, t - 1]
+    for extra in np.linspace(0, t - 1, want).astype(int):
+        if len(set(picks)) >= want:
+            break
+        picks.append(int(extra))
+    return sorted(set(picks)), busiest, len(singles)
+
+
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K"])
+def test_prefill_config_512_tokens_zipf(cuda, fmt):
+    """Benchmark prefill configuration: T=512, Zipf(1.1) routing, in the three formats the benchmark
+    times.  Routing of every token against the oracle; outputs of 32 tokens chosen to cover the
+    busiest expert's first / middle / last chunk, a one-token expert and the first and last expert
+    in use against the oracle; and, size-independent, a token's output equals the same token run
+    alone (dispatch and compaction are permutation-invariant)."""
+    announce("moe prefill T=512", fmt)
     e, d, f, fsh, k, t = 512, 2048, 512, 2048, 10, 512
-    gate, up, down, shared, gate_vec, bank, dshared = full_layer("Q8_0", cuda)
-    hidden = synthetic.activations((t, d), 7, "bf16")
+    gate, up, down, shared, gate_vec, bank, dshared = full_layer(fmt, cuda)
+    # (the synthetic Q5_K minima make outputs large: same scale as the other Q5_K cases)
+    hidden = synthetic.activations((t, d), 7, "bf16") * np.float32(1.0 if fmt != "Q5_K" else 2.0 ** -6)
     logits = synthetic.router_logits(t, e, 9, zipf=1.1)
     assert not synthetic.has_topk_ties(logits, k)
     hd, ld, gd = torch.from_numpy(hidden).to(cuda), torch.from_numpy(logits).to(cuda), torch.from_numpy(gate_vec).to(cuda)
     out, w, ids = moe_step(hd, bank, k, logits=ld, shared=dshared, shared_gate=gd, return_routing=True)
-    counts = np.bincount(ids.cpu().numpy().ravel(), minlength=e)
+    ids_host = ids.cpu().numpy()
+    want_w_all, want_ids_all = R.router_topk(logits, k, renormalize=True, floor=2.0 ** -14)
+    np.testing.assert_array_equal(ids_host, want_ids_all)
+    np.testing.assert_allclose(w.cpu().numpy(), want_w_all, rtol=2e-6, atol=2e-7)
+    counts = np.bincount(ids_host.ravel(), minlength=e)
     assert counts.max() > 5 * counts.mean()  # the routing really is skewed
-    picks = [0, 17, 255, 511]
-    for i in picks:
+    picks, busiest, n_single = prefill_sample(ids_host, e)
+    assert len(picks) >= 32 and counts[busiest] > 64
+    for i in (picks[0], picks[len(picks) // 2], picks[-1]):
         alone = moe_step(hd[i:i + 1].contiguous(), bank, k, logits=ld[i:i + 1].contiguous(), shared=dshared, shared_gate=gd)
         assert rel_l2(out[i:i + 1].cpu().numpy(), alone.cpu().numpy()) <= 1e-5
-    want, _, want_ids = oracle_step(hidden[picks[:2]], logits[picks[:2]], k, gate, up, down, shared, gate_vec)
-    np.testing.assert_array_equal(ids.cpu().numpy()[picks[:2]], want_ids)
-    assert rel_l2(out.cpu().numpy()[picks[:2]], want) <= 2e-5
+    want, _, want_ids = oracle_step(hidden[picks], logits[picks], k, gate, up, down, shared, gate_vec)
+    np.testing.assert_array_equal(ids_host[picks], want_ids)
+    got = out.cpu().numpy()[picks]
+    assert rel_l2(got, want) <= 2e-5
+    for row in range(len(picks)):
+        assert rel_l2(got[row], want[row]) <= 5e-5, picks[row]
 
 
 @pytest.mark.parametrize("fmt", ["Q8_0", "BF16"])
