@@ -216,7 +216,54 @@ def cpu_baseline(budget_s=24.0):
             "seconds_total": round(time.perf_counter() - t_begin, 1), "numpy": np.__version__, "host_cpus": os.cpu_count()}
 
 
-def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=False, hot=False):
+TIMELINE_STAMPS = {
+    0: ("route + gate/up kernel", ["wave enters", "token routed / activations staged", "",
+                                   "at the barrier", "past the barrier", "first item's rows arrived", "wave ends"]),
+    1: ("down kernel", ["wave enters", "routing arrived, two rows requested", "activations arrived", "past the barrier",
+                        "first row arrived", "wave ends", "(routing arrived)", "(row addresses ready)"]),
+}
+
+
+def read_timeline(lib, steps_fn, steps):
+    """Per-phase timeline of the two MoE decode kernels from a library built with time stamps
+    (python -m mylocal_llm_amd._build --timeline): one step at a time, stamps read back after each;
+    microseconds after the first wave of the first kernel entered, min / mean / max over the waves
+    that wrote the stamp, averaged over the steps."""
+    import numpy as np
+    if not hasattr(lib, "qmoe_timeline_read"):
+        raise RuntimeError("this library was built without time stamps: build with `python -m mylocal_llm_amd._build --timeline` "
+                           "and set QMOE_LIBRARY to mylocal_llm_amd/libqmoe_hip_timeline.so")
+    lib.qmoe_timeline_read.argtypes = [ctypes.c_void_p]
+    buf = np.zeros((2, 4096, 8), dtype=np.uint64)
+    acc = {}
+    for _ in range(steps):
+        buf[:] = 0
+        # clear the device copy by reading after a step only: stamps are rewritten by every wave of every launch
+        steps_fn()
+        if lib.qmoe_timeline_read(buf.ctypes.data):
+            raise RuntimeError("qmoe_timeline_read failed")
+        t0 = buf[0, :, 0][buf[0, :, 0] > 0].min()
+        for kernel, (_, names) in TIMELINE_STAMPS.items():
+            for i, name in enumerate(names):
+                if not name:
+                    continue
+                col = buf[kernel, :, i]
+                col = col[col >= t0].astype(np.float64)
+                if col.size:
+                    us = (col - float(t0)) / 100.0
+                    acc.setdefault((kernel, i), []).append((us.min(), us.mean(), us.max(), col.size))
+    out = []
+    for kernel, (kname, names) in TIMELINE_STAMPS.items():
+        for i, name in enumerate(names):
+            rows = acc.get((kernel, i)) if name else None
+            if rows:
+                a = np.asarray(rows)
+                out.append({"kernel": kname, "stamp": name, "waves": int(a[:, 3].mean()), "min_us": round(a[:, 0].mean(), 2),
+                            "mean_us": round(a[:, 1].mean(), 2), "max_us": round(a[:, 2].mean(), 2)})
+    return out
+
+
+def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=False, hot=False, timeline=False):
     """512-expert top-10 MoE decode step (D=2048, F=512, shared F=2048).
 
     Cold (the default, the figure a model with dozens of layers sees): steps rotate over four
@@ -286,6 +333,13 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=
         if rc:
             raise RuntimeError(lib.qmoe_last_error().decode())
 
+    if timeline:
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for _ in range(warmup):
+            fn(stream)
+        torch.cuda.synchronize()
+        return {"workload": f"moe_decode_{fmt}_T{tokens} timeline", "unit": "us after the first wave entered the first kernel",
+                "stamps": read_timeline(lib, lambda: fn(stream), steps)}
     wall, ms = time_steps(torch, fn, steps, warmup)
     # algorithmic bytes: distinct selected experts (averaged over the steps actually run) + shared expert
     used = sorted({j % cycle for j in range(warmup, warmup + steps)})
@@ -415,7 +469,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_layer_half", "layer_few_tokens", "read_probe",
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_timeline", "moe_layer_half", "layer_few_tokens", "read_probe",
                                        "layer_q6_k", "layer_q5_k", "layer_q4_k", "layer_by_dependency"], default=None,
                     help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -440,6 +494,9 @@ def main():
         return
     if args.only == "moe_decode":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup) for t in (1, 4, 16)]))
+        return
+    if args.only == "moe_timeline":
+        print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, timeline=True) for t in (1, 4)], indent=1))
         return
     if args.only == "moe_decode_hot":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, hot=True) for t in (1, 4, 16)]))

@@ -80,7 +80,9 @@ _LIB = None
 
 
 def library_path():
-    return _build.LIB_PATH
+    """The library this process binds: QMOE_LIBRARY names another build of it (the measurement
+    variant with time stamps, say), otherwise the one built in-tree."""
+    return os.environ.get("QMOE_LIBRARY") or _build.LIB_PATH
 
 
 def load():

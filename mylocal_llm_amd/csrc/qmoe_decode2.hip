@@ -1,0 +1,882 @@
+// Packed-expert MoE decode step, rows through LDS by LDS-DMA: the two launches of a step of a few
+// tokens, written for the case where a launch is a handful of microseconds long and every phase of
+// it is a memory round trip.  Both kernels run one workgroup of eight waves per CU and fetch
+// weight rows with global_load_lds_dwordx4 (consecutive lanes, consecutive 16 bytes, straight into
+// LDS: no register holds a byte in flight, every cache line is requested once), so a wave can put
+// everything it will need in flight the moment it knows the addresses.
+//
+//   pairs2_kernel   routing + gate/up, up to four tokens.  The first T waves of every workgroup
+//                   route a token each; the other waves meanwhile stage the tokens' activations
+//                   and request and multiply rows of the shared expert, which need no routing.
+//                   After the workgroup's one barrier all waves walk the item stream (shared
+//                   expert rows first, then token by token the selected experts) through a ring
+//                   of LDS slots.  A slot holds the gate rows of an item in its first half and the
+//                   up rows in its second, so one pass of a wave over a slot yields silu(g) * u.
+//   down2_kernel    down projection, ordered combine, shared expert, residual: up to sixteen
+//                   tokens.  A wave owns one or two output rows for ALL tokens: the shared
+//                   expert's row is fetched once, the selected experts' rows token after token
+//                   into a two-deep ring, and the token's SwiGLU activations are staged once per
+//                   workgroup by DMA.  Lanes are laid out [expert slot][row part] plus a group for
+//                   the shared expert; the wave adds the products in ascending expert id (product
+//                   rounded, then added) and finally shared * sigmoid.
+//
+// The kernels' waits are counted by hand (s_waitcnt vmcnt with the number of newer requests), so
+// every global load in them is either a DMA or an inline-assembly load whose result is not
+// touched before the wait that covers it; stores only make those waits conservative.
+#include "qmoe_decode.hpp"
+#include "qmoe_rowdot.hpp"
+#include "qmoe_span.hpp"
+
+namespace qmoe {
+
+static constexpr int D2_WAVES = 8;
+static constexpr int D2_THREADS = D2_WAVES * 64;
+static constexpr int D2_LDS = 160 * 1024;
+
+// Per-wave time stamps of the two kernels' phases, for builds with -DQMOE_TIMELINE only (the
+// measurement build of `python -m mylocal_llm_amd._build --timeline`; bench.py --only moe_timeline
+// reads them): stamp i of wave w of kernel k is the 100 MHz device counter when the wave got there.
+#ifdef QMOE_TIMELINE
+static constexpr int TL_WAVES = 4096, TL_STAMPS = 8;
+static __device__ unsigned long long timeline[2][TL_WAVES][TL_STAMPS];
+#define QMOE_STAMP(kernel, index)                                                                          \
+    do {                                                                                                   \
+        const int w_ = blockIdx.x * D2_WAVES + (threadIdx.x >> 6);                                         \
+        if ((threadIdx.x & 63) == 0 && w_ < TL_WAVES) timeline[kernel][w_][index] = wall_clock64();        \
+    } while (0)
+#else
+#define QMOE_STAMP(kernel, index) ((void)0)
+#endif
+
+// 16 bytes per lane from a per-lane 64-bit address into LDS at m0 + 16 lane.
+__device__ __forceinline__ void dma16_at(const uint8_t* lane_address) {
+    asm volatile("global_load_lds_dwordx4 %0, off" ::"v"(lane_address) : "memory");
+}
+// 4 bytes per lane into LDS at m0 + 4 lane
+__device__ __forceinline__ void dma4_at(const void* lane_address) {
+    asm volatile("global_load_lds_dword %0, off" ::"v"(lane_address) : "memory");
+}
+// ... on the lanes of `mask` only (a wave-uniform 64-bit lane mask, not zero)
+__device__ __forceinline__ void dma16_at_masked(const uint8_t* lane_address, uint64_t mask) {
+    uint64_t save;
+    mask = ((uint64_t)(uint32_t)uniform((int)(mask >> 32)) << 32) | (uint32_t)uniform((int)(uint32_t)mask);
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(save) : "v"(lane_address), "s"(mask) : "memory");
+}
+// One dword per lane; the result must not be touched before a wait that covers the load
+// (settle() names the values such a wait has released).
+__device__ __forceinline__ uint32_t load_u32_unwaited(const void* lane_address) {
+    uint32_t v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(lane_address) : "memory");
+    return v;
+}
+__device__ __forceinline__ void settle(uint32_t& a) { asm volatile("" : "+v"(a)::"memory"); }
+__device__ __forceinline__ u32x2_t load_u32x2_unwaited(const void* lane_address) {
+    u32x2_t v;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(lane_address) : "memory");
+    return v;
+}
+__device__ __forceinline__ u32x4_t load_u32x4_unwaited(const void* lane_address) {
+    u32x4_t v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(lane_address) : "memory");
+    return v;
+}
+__device__ __forceinline__ void settle(u32x2_t& a) { asm volatile("" : "+v"(a)::"memory"); }
+__device__ __forceinline__ void settle(u32x4_t& a) { asm volatile("" : "+v"(a)::"memory"); }
+
+// s_waitcnt vmcnt(n) for a wave-uniform n known only at run time (the count is an immediate).
+__device__ __forceinline__ void wait_vmcnt_rt(int n) {
+    switch (n) {
+#define QMOE_W(N) case N: wait_vmcnt<N>(); break;
+        QMOE_W(1) QMOE_W(2) QMOE_W(3) QMOE_W(4) QMOE_W(5) QMOE_W(6) QMOE_W(7) QMOE_W(8) QMOE_W(9) QMOE_W(10)
+        QMOE_W(11) QMOE_W(12) QMOE_W(13) QMOE_W(14) QMOE_W(15) QMOE_W(16) QMOE_W(17) QMOE_W(18) QMOE_W(19) QMOE_W(20)
+        QMOE_W(21) QMOE_W(22) QMOE_W(23) QMOE_W(24) QMOE_W(25) QMOE_W(26) QMOE_W(27) QMOE_W(28) QMOE_W(29) QMOE_W(30)
+#undef QMOE_W
+    default: wait_vmcnt<0>(); break;
+    }
+}
+
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+    const uint32_t lo = (uint32_t)uniform((int)(uint32_t)v), hi = (uint32_t)uniform((int)(uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Sum over groups of `lpe` consecutive lanes (1, 2, 4, 8 or 16), the total in every lane of a group.
+__device__ __forceinline__ float part_sum_rt(float v, int lpe) {
+    if (lpe >= 2) v = dpp_add<0xB1>(v);
+    if (lpe >= 4) v = dpp_add<0x4E>(v);
+    if (lpe >= 8) v = dpp_add<0x141>(v);
+    if (lpe >= 16) v = dpp_add<0x140>(v);
+    return v;
+}
+
+// ================================================================================================
+// down projection
+// ================================================================================================
+static constexpr int DOWN2_MAX_TOKENS = 16;
+static constexpr int DOWN2_CI = 8, DOWN2_CH = 4;   // most DMA instructions per row image / per wave for the activations
+
+struct Down2Args {
+    const uint8_t* down;         // bank base, [E, D, F]
+    int64_t down_stride;
+    const uint8_t* shared_down;  // [D, Fsh] or null
+    const float* h;              // [T*k, F] in sorted-slot order
+    const float* hs;             // [T, Fsh]
+    const int* sorted_ids;       // [T, k]
+    const float* sorted_w;       // [T, k]
+    const float* sig;            // [T]
+    void* out;                   // [T, D]
+    const float* residual;       // [T, D] or null
+    int odt, k, d, f, fsh;
+    int rows;                    // output rows per wave
+    int lpe;                     // lanes per expert row: f / 128
+    int ppr, pps;                // 16-byte pieces of the LDS image of one routed row / of the shared row
+    uint32_t ppr_magic;          // floor(2^32 / ppr) + 1: p / ppr by mulhi, exact for the few hundred pieces of an image
+    int ci, ch;                  // DMA instructions per row image, per wave for the activations
+    int image;                   // LDS bytes of a row image: the k routed rows, then the shared row
+    int hbytes;                  // LDS bytes of the staged activations, whole KB
+};
+
+// One workgroup = one token x 8 waves x `rows` output rows.  A row's image -- row r of each of the
+// token's k experts, then row r of the shared expert -- is one request (DMA instructions of 64
+// pieces, the last one on the lanes that are left); a wave keeps two images in flight: as soon as
+// an image's bytes are in registers its slot is requested into again, so two rows are on their way
+// while one is multiplied.
+// LDS: [staged activations | per wave: expert ids | dump | per wave: two row images]
+template <int FMT>
+__global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a) {
+    using U = Unit64<FMT>;
+    using S = SpanFmt<FMT>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63, wave = uniform((int)(threadIdx.x >> 6));
+    const int k = a.k, R = a.rows, t = blockIdx.y;
+    uint8_t* const hbuf = lds;
+    int* const tab_ids = (int*)(lds + a.hbytes + wave * 768);   // this wave's copy of the token's routing: 64 ids,
+    float* const tab_w = (float*)(tab_ids + 64);                 // 64 weights, the sigmoid gate (entries past k repeat entry k - 1)
+    float* const tab_sig = tab_w + 64;
+    uint8_t* const dump = lds + a.hbytes + D2_WAVES * 768;
+    uint8_t* const ring = dump + 1024 + wave * (2 * a.image);
+    const int row0 = (blockIdx.x * D2_WAVES + wave) * R;   // first output row of this wave
+    const int64_t rb_r = row_bytes_dev(FMT, a.f), rb_s = row_bytes_dev(FMT, a.fsh);
+    auto clamp_row = [&](int i) { return row0 + i < a.d ? row0 + i : a.d - 1; };
+    QMOE_STAMP(1, 0);
+
+    // ---- 1. the token's routing, by DMA into this wave's table (no register waits for a load) ------
+    const int kk = lane < k ? lane : k - 1;
+    set_m0((uint32_t)(uintptr_t)tab_ids);
+    dma4_at(a.sorted_ids + t * k + kk);
+    set_m0((uint32_t)(uintptr_t)tab_w);
+    dma4_at(a.sorted_w + t * k + kk);
+    set_m0((uint32_t)(uintptr_t)tab_sig);
+    dma4_at(a.sig + t);
+
+    // ---- 2. the token's activations: [h of its k slots | hs], swizzled while they travel --------
+    // LDS granule P = 64 chunk + lane receives source granule swizzled(P); a wave brings chunks
+    // wave, wave + 8, ...; chunks past the end fetch into the dump.
+    const int nr = k * a.f, n_gran = (nr + (a.shared_down ? a.fsh : 0)) >> 2;
+    {
+        const uint8_t* const hr = (const uint8_t*)(a.h + (size_t)t * nr);
+        const uint8_t* const hsr = (const uint8_t*)(a.hs + (size_t)t * a.fsh);
+#pragma unroll
+        for (int i = 0; i < DOWN2_CH; ++i)
+            if (i < a.ch) {
+                const int chunk = wave + D2_WAVES * i;
+                const int P = 64 * chunk + lane;
+                const int g = swizzled_granule(P);
+                const bool valid = P < n_gran, from_hs = valid && 4 * g >= nr;
+                const uint32_t off = valid ? (uint32_t)(from_hs ? 4 * g - nr : 4 * g) * 4u : 0u;
+                set_m0((uint32_t)(uintptr_t)(64 * chunk < n_gran ? hbuf + 1024 * chunk : dump));
+                dma16_at(from_hs ? hsr + off : hr + off);
+            }
+    }
+
+    // ---- 3. the routing into registers and LDS ----------------------------------------------------
+    wait_vmcnt_rt(a.ch);
+    QMOE_STAMP(1, 6);
+    const float route_w = lane < k ? tab_w[lane] : 0.f;   // lane j holds weight j
+    const float sg = tab_sig[0];
+
+    // ---- 4. where piece p = lane + 64 c of a row image comes from ---------------------------------
+    // p < k ppr: piece p % ppr of expert slot p / ppr; then the pieces of the shared row.
+    // With a residual, one more piece: the 16 bytes that hold the residual's value of the row (an
+    // ordinary load here would make the compiler wait for everything in flight).
+    const uint8_t* src[DOWN2_CI];
+    uint32_t is_shared = 0, is_residual = 0;
+    const int routed_pieces = k * a.ppr, weight_pieces = routed_pieces + a.pps, pieces = weight_pieces + (a.residual ? 1 : 0);
+#pragma unroll
+    for (int c = 0; c < DOWN2_CI; ++c) {
+        const int p = lane + 64 * c;
+        const uint8_t* from = a.down;
+        if (p < routed_pieces) {
+            const int j = (int)__umulhi((uint32_t)p, a.ppr_magic), q = p - j * a.ppr;
+            const int e = tab_ids[j];
+            from = a.down + (int64_t)(e >= 0 ? e : 0) * a.down_stride + S::src(q);
+        } else if (p < weight_pieces) {
+            from = a.shared_down + S::src(p - routed_pieces);
+            is_shared |= 1u << c;
+        } else if (p < pieces) {
+            from = (const uint8_t*)(a.residual + (size_t)t * a.d);
+            is_residual |= 1u << c;
+        }
+        src[c] = from;
+    }
+    const int last_lanes = pieces - 64 * (a.ci - 1);   // lanes of the last instruction, 1..64
+    const uint64_t last_mask = last_lanes >= 64 ? ~0ull : ((1ull << last_lanes) - 1);
+    auto request = [&](int i) {   // row i of this wave into slot i & 1
+        const int row = clamp_row(i);
+        const int64_t at_r = (int64_t)row * rb_r, at_s = (int64_t)row * rb_s, at_res = (int64_t)(row & ~3) * 4;
+        uint8_t* const img = ring + (i & 1) * a.image;
+#pragma unroll
+        for (int c = 0; c < DOWN2_CI; ++c)
+            if (c < a.ci) {
+                const uint8_t* const from = src[c] + (((is_shared >> c) & 1u) ? at_s : ((is_residual >> c) & 1u) ? at_res : at_r);
+                set_m0((uint32_t)(uintptr_t)(img + 1024 * c));
+                if (c + 1 < a.ci) dma16_at(from);
+                else dma16_at_masked(from, last_mask);
+            }
+    };
+    const int per_request = a.ci;
+    QMOE_STAMP(1, 7);
+    request(0);
+    if (R > 1) request(1);
+    QMOE_STAMP(1, 1);
+
+    // ---- lane layout of the multiplication -------------------------------------------------------
+    const int lpe = a.lpe;
+    const int shared_parts = a.shared_down ? a.fsh >> 7 : 0;
+    const bool routed = lane < k * lpe;
+    const bool shared = lane >= 48 && lane - 48 < shared_parts;
+    const int slot = routed ? lane / lpe : 0;
+    const int part = routed ? lane % lpe : (shared ? lane - 48 : 0);
+    const int ux = shared ? (nr >> 6) + 2 * part : slot * (a.f >> 6) + 2 * part;
+    const uint32_t row_at = shared ? routed_pieces * 16 : slot * a.ppr * 16;
+    const uint32_t unit_at0 = row_at + S::unit_offset(2 * part), unit_at1 = row_at + S::unit_offset(2 * part + 1);
+    const bool live = (routed && tab_ids[slot] >= 0) || shared;
+
+    // the activations have arrived (this wave's share; the barrier covers the others')
+    wait_vmcnt_rt((R > 1 ? 2 : 1) * per_request);
+    QMOE_STAMP(1, 2);
+    __syncthreads();
+    QMOE_STAMP(1, 3);
+    float x0[64], x1[64], aux0[U::AUX], aux1[U::AUX];
+    U::load_x(SwizzledX{hbuf}, ux, x0, aux0);
+    U::load_x(SwizzledX{hbuf}, ux + 1, x1, aux1);
+
+    for (int i = 0; i < R; ++i) {
+        if (i + 1 < R) wait_vmcnt_rt(per_request);
+        else wait_vmcnt<0>();
+        if (i == 0) QMOE_STAMP(1, 4);
+        const uint8_t* const img = ring + (i & 1) * a.image;
+        uint32_t r0[U::RAW], r1[U::RAW];
+        S::read(img + unit_at0, 2 * part, r0);
+        S::read(img + unit_at1, 2 * part + 1, r1);
+        const float before = a.residual ? *(const float*)(img + weight_pieces * 16 + ((row0 + i) & 3) * 4) : 0.f;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the image is in registers: its slot is free
+        if (i + 2 < R) request(i + 2);
+        float v = U::dot(r0, x0, aux0) + U::dot(r1, x1, aux1);
+        if (!live) v = 0.f;   // idle lanes decoded whatever lies at the start of the image
+        const float ys = group_sum<16>(v);      // lanes 48..63 are one DPP row: the shared expert's total
+        const float yr = part_sum_rt(v, lpe);   // every slot's total in each of its lanes
+        float acc = 0.f;
+        for (int j = 0; j < k; ++j) {
+            const float yj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(yr), j * lpe));
+            const float wj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(route_w), j));
+            acc = add_product(acc, yj, wj);
+        }
+        if (a.shared_down) {
+            const float y63 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ys), 63));
+            acc = add_product(acc, y63, sg);
+        }
+        const int row = row0 + i;
+        if (lane == 0 && row < a.d) {
+            if (a.residual) acc = before + acc;
+            store_out(a.out, a.odt, (size_t)t * a.d + row, acc);
+        }
+    }
+    QMOE_STAMP(1, 5);
+}
+
+// ================================================================================================
+// routing + gate/up
+// ================================================================================================
+static constexpr int PAIRS2_MAX_TOKENS = 4;
+static constexpr int PAIRS2_MAX_EXPERTS = 1024;   // two router values per lane at most when eight waves share a row
+static constexpr int PAIRS2_MAX_K = 16;
+static constexpr int PAIRS2_PD = 2;               // slots requested ahead of the one being multiplied
+static constexpr int PAIRS2_NV = 8;               // most router values per lane
+
+struct Pairs2Shape {
+    int lr;            // lanes per row (8, 16 or 32)
+    int ri;            // rows of an item: 32 / lr (a slot holds ri gate rows, then the same ri up rows)
+    int row_image;     // LDS bytes of one row's image
+    int pph;           // 16-byte pieces of half a slot: ri rows
+    int ipe, ish;      // items per expert pair (f / ri), of the shared pair (fsh / ri)
+    int total;         // ish + tokens * k * ipe
+    uint32_t ipe_magic, k_magic;   // floor(2^32 / d) + 1: exact quotients by mulhi for the sizes taken here
+    int xs_bytes;      // LDS bytes of the staged activations (tokens * d * 4)
+    int gw;            // waves that route one token together: 8, 4 or 2
+    int nv;            // router values per lane: ceil(n_experts / (64 gw))
+};
+
+// What the waves that route one token together leave for each other in LDS.
+struct RouteShare {
+    uint32_t max_key[D2_WAVES];
+    uint32_t has_nan[D2_WAVES];
+    double partial[D2_WAVES];
+    uint32_t cand_key[D2_WAVES * PAIRS2_MAX_K];   // each wave's own best k, best first
+    int cand_id[D2_WAVES * PAIRS2_MAX_K];
+};
+
+// The best k of one wave's stretch of a router row (NV values per lane, value j of a lane is expert
+// id0 + lane + 64 j): lane s < k receives the s-th best as (order key, expert id); the stretch's best
+// key and whether it holds a NaN come back for the row's maximum.  Keys: order_key with every NaN
+// raised to 1 (below -inf, above 0 = "taken or absent"); ties go to the lower id.
+template <int NV>
+__device__ __forceinline__ void stretch_best(const float* v, int id0, int n, int k, uint32_t& wave_best, bool& any_nan,
+                                             uint32_t& my_key, int& my_id) {
+    const int lane = threadIdx.x & 63;
+    uint32_t key[NV];
+    uint32_t best = 0u;
+    bool nan_seen = false;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const bool valid = id0 + lane + 64 * j < n;
+        const uint32_t ok = order_key(v[j]);
+        key[j] = valid ? (ok ? ok : 1u) : 0u;
+        nan_seen |= valid && ok == 0u;
+        best = key[j] > best ? key[j] : best;
+    }
+    wave_best = wave_max_u32(best);
+    any_nan = __any(nan_seen);
+    for (int slot = 0; slot < k; ++slot) {
+        uint32_t c = 0u;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) c = key[j] > c ? key[j] : c;
+        const uint32_t win = wave_max_u32(c);
+        int wj = -1;   // owner: first j with a holder, then the lowest lane holding it there
+        unsigned long long holders = 0ull;
+#pragma unroll
+        for (int j = NV - 1; j >= 0; --j) {
+            const unsigned long long b = __ballot(key[j] == win);
+            if (b) { wj = j; holders = b; }
+        }
+        const int wl = __builtin_ctzll(holders);
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            if (j == wj) key[j] = lane == wl ? 0u : key[j];
+        if (lane == slot) { my_key = win; my_id = id0 + wl + 64 * wj; }
+    }
+}
+
+template <int FMT> struct Pairs2Slot {
+    static constexpr int CH = SpanSlot<FMT>::CHUNKS;    // DMA instructions per slot
+    static constexpr int BYTES = CH * 1024;             // (whole instructions: no lane mask)
+};
+
+// LDS: [activations fp32, swizzled | sorted ids per token | dump | rings: 8 waves x 3 slots]
+template <int FMT>
+__global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRouteArgs a, const Pairs2Shape x) {
+    using U = Unit64<FMT>;
+    using S = SpanFmt<FMT>;
+    using SL = Pairs2Slot<FMT>;
+    constexpr int PD = PAIRS2_PD, NS = PD + 1, CH = SL::CH;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63, wave = uniform((int)(threadIdx.x >> 6));
+    const int T = a.tokens, k = a.k;
+    uint8_t* const xs = lds;
+    int64_t* const sid = (int64_t*)(lds + x.xs_bytes);                  // [PAIRS2_MAX_TOKENS][32]
+    uint8_t* const dump = (uint8_t*)(sid + PAIRS2_MAX_TOKENS * 32) + PAIRS2_MAX_TOKENS * sizeof(RouteShare);
+    uint8_t* const ring = dump + 1024 + wave * (NS * SL::BYTES);
+    const int64_t rb = row_bytes_dev(FMT, a.d);
+    const int lr = x.lr, units = a.d >> 6;
+    const int u = lane & (lr - 1), sub = lane / lr;
+    const bool active = u < units;
+    const uint32_t lane_off = sub * x.row_image + S::unit_offset(active ? u : 0);
+
+    // where piece p = lane + 64 c of a slot comes from: half (gate / up rows) and offset inside it
+    uint32_t p_off[CH];
+    uint32_t p_up = 0;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int p = lane + 64 * c;
+        const bool up = p >= x.pph, valid = p < 2 * x.pph;
+        p_off[c] = valid ? (uint32_t)S::src(up ? p - x.pph : p) : 0u;
+        p_up |= (up && valid ? 1u : 0u) << c;
+    }
+
+    struct Item {
+        const uint8_t *g, *u;   // first gate / up row of the item
+        float* y;               // where row r0 of the result goes (token 0 of a shared item)
+        int t;                  // token, -1 for the shared expert (all tokens)
+        int r0;
+        bool live;
+    };
+    auto decode = [&](int g) {
+        Item it;
+        it.g = it.u = a.gate;
+        it.y = nullptr;
+        it.t = 0;
+        it.r0 = 0;
+        it.live = false;
+        if (g < x.ish) {
+            it.r0 = g * x.ri;
+            it.g = a.shared_gate_w + (int64_t)it.r0 * rb;
+            it.u = a.shared_up_w + (int64_t)it.r0 * rb;
+            it.y = a.hs + it.r0;
+            it.t = -1;
+            it.live = true;
+        } else if (g < x.total) {
+            const uint32_t q = (uint32_t)(g - x.ish);
+            const uint32_t tj = __umulhi(q, x.ipe_magic);
+            const uint32_t t = k == 1 ? tj : __umulhi(tj, x.k_magic);
+            it.r0 = (int)(q - tj * (uint32_t)x.ipe) * x.ri;
+            it.t = (int)t;
+            const int64_t e = uniform64(sid[t * 32 + (tj - t * (uint32_t)k)]);
+            if (e >= 0) {
+                it.g = a.gate + e * a.gate_stride + (int64_t)it.r0 * rb;
+                it.u = a.up + e * a.up_stride + (int64_t)it.r0 * rb;
+                it.y = a.h + (size_t)tj * a.f + it.r0;
+                it.live = true;
+            }
+        }
+        it.g = uniform(it.g);
+        it.u = uniform(it.u);
+        return it;
+    };
+    auto request = [&](int slot, const Item& it) {
+        uint8_t* const at = ring + slot * SL::BYTES;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            set_m0((uint32_t)(uintptr_t)(at + 1024 * c));
+            // (an item past the end fetches one line, sixty-four times the same 16 bytes)
+            dma16_at(it.live ? (((p_up >> c) & 1u) ? it.u + p_off[c] : it.g + p_off[c]) : it.g);
+        }
+    };
+    float xr[64], aux[8];
+    int held = -1;   // the token whose slice of the activations is in xr
+    auto multiply = [&](int slot, const Item& it) {
+        uint32_t r[U::RAW];
+        S::read(ring + slot * SL::BYTES + lane_off, u, r);
+        const int t0 = it.t < 0 ? 0 : it.t, t1 = it.t < 0 ? T : it.t + 1;
+        for (int t = t0; t < t1; ++t) {
+            if (held != t) {
+                U::load_x(SwizzledX{xs + (size_t)t * a.d * 4}, active ? u : 0, xr, aux);
+                held = t;
+            }
+            float v = U::dot(r, xr, aux);
+            v = group_sum_rt(active ? v : 0.f, lr);           // (a lane without a unit has read bytes of another one)
+            const float partner = __shfl_xor(v, 32, 64);      // the up row's total, for the lanes of the gate row
+            if (lane < 32 && u == lr - 1) {
+                float* const y = it.t < 0 ? it.y + (size_t)t * a.fsh : it.y;
+                stg<float>(y + sub, silu_mul(v, partner));
+            }
+        }
+    };
+
+    // ---- routing, activations, and a first row pair of the shared expert ---------------------------
+    // The waves of a workgroup route together: `gw` waves per token, each with its own stretch of
+    // the router row (one value per lane for 512 experts and one token).  A wave picks the best k of
+    // its stretch, the waves of a token exchange those through LDS, and each of them then picks the
+    // best k of the gw * k candidates by itself -- the same order keys, the same tie rule (lower id),
+    // so the result is the single-wave router's, in a fraction of its instructions.  Every load of
+    // this part is an inline-assembly load with a wait of its own: the row pair of the shared expert
+    // that a wave requests first must not be waited for by anything here.
+    QMOE_STAMP(0, 0);
+    const int n = a.n_experts;
+    const int group = wave / x.gw, wg = wave - group * x.gw;   // token `group`, position in its group
+    const bool routes = group < T;
+    const bool from_logits = a.logits != nullptr;
+    RouteShare* const share = (RouteShare*)(sid + PAIRS2_MAX_TOKENS * 32) + group;
+    // The waves that publish the routing (workgroup 0, the first wave of each token's group) take
+    // no items: they have the admission gate to compute, with ordinary loads, which must not meet
+    // requests in flight.  All other waves share the item stream.
+    const bool publishes = blockIdx.x == 0 && routes && wg == 0;
+    // (a) the routing given by the caller (ordinary loads, waited for before anything else is issued)
+    float weight = 0.f;
+    int64_t id = 0;
+    if (routes && !from_logits) {
+        const int kk = lane < k ? lane : k - 1;
+        id = a.in_ids[(size_t)group * k + kk];
+        weight = a.in_weights[(size_t)group * k + kk];
+        asm volatile("" ::"v"((uint32_t)id), "v"((uint32_t)((uint64_t)id >> 32)), "v"(weight) : "memory");
+    }
+    // ... or the wave's stretch of the router row.  Everything a wave fetches here goes to LDS by
+    // DMA (router values and 16-bit activations into the wave's own ring slots, which are free until
+    // the barrier; fp32 activations straight to their place), so that no register waits for a load.
+    const int id0 = wg * 64 * x.nv;   // first expert of this wave's stretch
+    uint8_t* const lds_logits = ring + SL::BYTES;       // value j of lane l at 256 j + 4 l
+    uint8_t* const lds_xraw = ring + 2 * SL::BYTES;     // this wave's 16-bit chunks, 512 bytes each
+    int n_loads = 0;
+    if (routes && from_logits) {
+        const float* const row = a.logits + (size_t)group * n;
+        for (int j = 0; j < x.nv; ++j) {
+            const int at = id0 + lane + 64 * j;
+            set_m0((uint32_t)(uintptr_t)(lds_logits + 256 * j));
+            dma4_at(row + (at < n ? at : n - 1));
+            ++n_loads;
+        }
+    }
+    const int n_logit_loads = n_loads;
+    // (b) this wave's share of the tokens' activations: 256-column chunks wave, wave + 8, ... of all tokens
+    const int per_token = a.d >> 8, chunks = T * per_token;
+    if (a.xdt == QMOE_DT_F32) {
+        for (int c = wave; c < chunks; c += D2_WAVES) {
+            const int t = c / per_token, cc = c - t * per_token;
+            // LDS granule 64 cc + lane receives source granule swizzled(64 cc + lane)
+            const float* const src = (const float*)a.hidden + (size_t)t * a.d + 4 * swizzled_granule(64 * cc + lane);
+            set_m0((uint32_t)(uintptr_t)(xs + (size_t)t * a.d * 4 + 1024 * cc));
+            dma16_at((const uint8_t*)src);
+            ++n_loads;
+        }
+    } else {
+        for (int q = 0; 2 * q * D2_WAVES + wave < chunks; ++q) {   // two chunks per instruction: lanes 0..31, 32..63
+            const int c = wave + D2_WAVES * (2 * q + (lane >> 5));
+            const uint16_t* const src = (const uint16_t*)a.hidden + 256 * (size_t)(c < chunks ? c : wave) + 8 * (lane & 31);
+            set_m0((uint32_t)(uintptr_t)(lds_xraw + 1024 * q));
+            dma16_at((const uint8_t*)src);
+            ++n_loads;
+        }
+    }
+    n_loads -= n_logit_loads;   // (requests newer than the router values)
+    // (c) a row pair of the shared expert, if the wave's first item is one
+    const int W = gridDim.x * D2_WAVES - T;                      // waves that take items
+    const int before = (wave + x.gw - 1) / x.gw;   // publishing waves of workgroup 0 ahead of this one
+    const int me = blockIdx.x * D2_WAVES + wave - (blockIdx.x == 0 ? (before < T ? before : T) : T);
+    const int g0 = publishes ? x.total : me;                      // this wave's items are g0, g0 + W, ...
+    const bool early = g0 < x.ish;   // the first item is a shared one, requested before the routing is known
+    Item it[NS];
+    if (early) {
+        it[0] = decode(g0);
+        request(0, it[0]);
+        n_loads += CH;
+    }
+    // (d) the wave's own best k
+    wait_vmcnt_rt(n_loads);
+    uint32_t my_key = 0u;
+    int my_id = 0;
+    float m = 0.f, denom = 1.f;
+    float v[PAIRS2_NV];
+#pragma unroll
+    for (int j = 0; j < PAIRS2_NV; ++j) v[j] = j < x.nv ? *(const float*)(lds_logits + 256 * j + 4 * lane) : 0.f;
+    if (routes && from_logits) {
+        uint32_t wave_best = 0u;
+        bool any_nan = false;
+        switch (x.nv) {
+        case 1: stretch_best<1>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
+        case 2: stretch_best<2>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
+        case 4: stretch_best<4>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
+        default: stretch_best<8>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
+        }
+        if (lane == 0) {
+            share->max_key[wg] = wave_best;
+            share->has_nan[wg] = any_nan ? 1u : 0u;
+        }
+        if (lane < k) {
+            share->cand_key[wg * k + lane] = my_key;
+            share->cand_id[wg * k + lane] = my_id;
+        }
+        QMOE_STAMP(0, 1);
+        __syncthreads();
+        // (e) the row's maximum, then this stretch's part of the softmax denominator
+        uint32_t row_best = 0u, row_nan = 0u;
+        for (int w2 = 0; w2 < x.gw; ++w2) {
+            const uint32_t o = share->max_key[w2];
+            row_best = o > row_best ? o : row_best;
+            row_nan |= share->has_nan[w2];
+        }
+        m = row_nan ? __uint_as_float(0x7FC00000u) : key_value(row_best);   // maximum with NaN propagation
+        double part = 0.0;
+#pragma unroll
+        for (int j = 0; j < PAIRS2_NV; ++j)
+            if (j < x.nv && id0 + lane + 64 * j < n) part += (double)expf(v[j] - m);
+        part = wave_sum_f64(part);
+        if (lane == 0) share->partial[wg] = part;
+    } else {
+        QMOE_STAMP(0, 1);
+        __syncthreads();
+    }
+    // (f) activations into LDS as fp32 (they have long arrived; only the row pair may still travel)
+    wait_vmcnt_rt(early ? CH : 0);
+    if (a.xdt != QMOE_DT_F32) {
+        for (int i = 0; wave + D2_WAVES * i < chunks; ++i) {
+            const int c = wave + D2_WAVES * i;
+            const uint2 w = *(const uint2*)(lds_xraw + 512 * i + 8 * lane);
+            float4 f;
+            if (a.xdt == QMOE_DT_BF16) {
+                f = make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xFFFF0000u),
+                                __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xFFFF0000u));
+            } else {
+                f = make_float4(__half2float(__ushort_as_half((unsigned short)(w.x & 0xFFFFu))), __half2float(__ushort_as_half((unsigned short)(w.x >> 16))),
+                                __half2float(__ushort_as_half((unsigned short)(w.y & 0xFFFFu))), __half2float(__ushort_as_half((unsigned short)(w.y >> 16))));
+            }
+            const int t = c / per_token, gran = 64 * (c - t * per_token) + lane;
+            *(float4*)(xs + (size_t)t * a.d * 4 + 16 * swizzled_granule(gran)) = f;
+        }
+    }
+    __syncthreads();
+    // (g) every wave of a token's group picks the best k of the group's candidates by itself
+    if (routes && from_logits) {
+        double total = 0.0;
+        for (int w2 = 0; w2 < x.gw; ++w2) total += share->partial[w2];
+        denom = (float)total;
+        const int cands = x.gw * k;   // candidate i = wave i / k, its rank i % k: ties fall to the lower id as before
+        uint32_t ck[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) ck[j] = lane + 64 * j < cands ? share->cand_key[lane + 64 * j] : 0u;
+        uint32_t sel_key = 0u;
+        int sel_at = 0;
+        for (int slot = 0; slot < k; ++slot) {
+            const uint32_t c = ck[0] > ck[1] ? ck[0] : ck[1];
+            const uint32_t win = wave_max_u32(c);
+            const unsigned long long b0 = __ballot(ck[0] == win), b1 = __ballot(ck[1] == win);
+            const int wj = b0 ? 0 : 1;
+            const int wl = __builtin_ctzll(b0 ? b0 : b1);
+            if (wj == 0) ck[0] = lane == wl ? 0u : ck[0];
+            else ck[1] = lane == wl ? 0u : ck[1];
+            if (lane == slot) { sel_key = win; sel_at = wl + 64 * wj; }
+        }
+        id = lane < k ? share->cand_id[sel_at] : 0;
+        // probabilities in parallel; their sum in selection order
+        const float p = lane < k ? expf(key_value(sel_key) - m) / denom : 0.0f;
+        float mass = 0.0f;
+        for (int slot = 0; slot < k; ++slot) mass += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), slot));
+        float norm = 1.0f;
+        if (a.renorm) norm = isnan(mass) ? mass : fmaxf(mass, a.floor_value);
+        weight = a.renorm ? p / norm : p;
+    }
+    if (routes) {
+        // rank of a selection in ascending expert id; equal ids keep slot order.  An id outside the
+        // bank, or an expert the token has named in an earlier slot already, contributes nothing.
+        int rank = 0;
+        bool again = false;
+        for (int j = 0; j < k; ++j) {
+            const int64_t other = readlane_i64(id, j);
+            rank += (other < id) || (other == id && j < lane);
+            again |= other == id && j < lane;
+        }
+        if (lane < k) {
+            const bool in_range = id >= 0 && id < n, ok = in_range && !again;
+            sid[group * 32 + rank] = ok ? id : -1;   // (every wave of the group writes the same values)
+            if (publishes) {        // one wave publishes the routing for the down kernel and the caller
+                if (!ok && a.status_out) atomicOr(a.status_out, (in_range ? 0 : 1) | (again ? 2 : 0));
+                if (a.out_weights) {
+                    a.out_weights[(size_t)group * k + lane] = weight;
+                    a.out_ids[(size_t)group * k + lane] = id;
+                }
+                a.sorted_ids[(size_t)group * k + rank] = ok ? (int)id : -1;
+                a.sorted_w[(size_t)group * k + rank] = weight;
+            }
+        }
+    }
+    QMOE_STAMP(0, 3);
+    __syncthreads();
+    QMOE_STAMP(0, 4);
+    // the sigmoid admission gate of the shared expert, by the publishing waves (which request nothing
+    // and end here), from the staged rows
+    if (publishes) {
+        float adm = 0.f;
+        if (a.shared_gate) {
+            for (int c = lane; c < (a.d >> 2); c += 64) {
+                const float4 h = *(const float4*)(xs + (size_t)group * a.d * 4 + 16 * swizzled_granule(c));
+                const float4 gv = ldg<float4>(a.shared_gate + 4 * c);
+                adm += (h.x * gv.x + h.y * gv.y) + (h.z * gv.z + h.w * gv.w);
+            }
+            adm = wave_sum(adm);
+        }
+        // sigmoid(hidden . g) without overflow
+        if (lane == 0) a.sig[group] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
+        return;
+    }
+
+    // ---- the item stream through the ring --------------------------------------------------------
+    int g = g0;
+    if (g >= x.total) return;   // (only where there are fewer items than waves: such a wave has requested nothing)
+#pragma unroll
+    for (int j = 0; j < PD; ++j)
+        if (j > 0 || !early) {
+            it[j] = decode(g + j * W);
+            request(j, it[j]);
+        }
+    bool done = false;
+    while (!done) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (!done) {
+                const int nb = (s + PD) % NS;
+                it[nb] = decode(g + PD * W);
+                request(nb, it[nb]);
+                wait_vmcnt<PD * CH>();
+                if (g == g0) QMOE_STAMP(0, 5);
+                if (it[s].live) multiply(s, it[s]);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the slot may be requested into again
+                g += W;
+                if (g >= x.total) done = true;
+            }
+        }
+    }
+    wait_vmcnt<0>();
+    QMOE_STAMP(0, 6);
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+static bool span_format(int fmt) {
+    return fmt == QMOE_FMT_Q8_0 || fmt == QMOE_FMT_Q6_K || fmt == QMOE_FMT_Q5_K || fmt == QMOE_FMT_Q4_K;
+}
+static int pieces_per_256(int fmt) {
+    return fmt == QMOE_FMT_Q8_0 ? 17 : fmt == QMOE_FMT_Q6_K ? 14 : fmt == QMOE_FMT_Q5_K ? 11 : 9;
+}
+static int kb(int bytes) { return (bytes + 1023) & ~1023; }
+
+static uint32_t magic_of(int d) { return (uint32_t)(0x100000000ull / (uint32_t)d) + 1u; }
+
+// Fills `out` if the down step of this MoE step is one down2_kernel takes.
+static bool down2_plan(const qmoe_moe_args& m, const DecodeBuffers& w, int cus, Down2Args* out) {
+    const qmoe_expert_bank& b = m.bank;
+    const bool has_shared = m.shared_down_w != nullptr;
+    if (!span_format(b.down_fmt) || (has_shared && m.shared_down_fmt != b.down_fmt)) return false;
+    if (m.tokens < 1 || m.tokens > DOWN2_MAX_TOKENS || m.tokens > cus || m.top_k > 16) return false;
+    const int lpe = b.d_ff >> 7;
+    if (b.d_ff % 256 || (lpe & (lpe - 1)) || lpe > 16 || m.top_k * lpe > 48) return false;
+    if (has_shared && (m.d_ff_shared % 256 || (m.d_ff_shared >> 7) > 16)) return false;
+    const int align = b.down_fmt == QMOE_FMT_Q6_K ? 2 : 16;
+    if ((uintptr_t)b.down % align || b.down_stride % align || (has_shared && (uintptr_t)m.shared_down_w % align)) return false;
+    if ((uintptr_t)w.h % 16 || (uintptr_t)w.hs % 16) return false;
+    Down2Args a{};
+    const int row_blocks = cus / m.tokens;   // workgroups per token
+    a.rows = (b.d_model + row_blocks * D2_WAVES - 1) / (row_blocks * D2_WAVES);
+    const int pp4 = pieces_per_256(b.down_fmt);
+    a.ppr = (b.d_ff >> 8) * pp4;
+    a.pps = has_shared ? (m.d_ff_shared >> 8) * pp4 : 0;
+    a.ppr_magic = magic_of(a.ppr);
+    if (m.residual && ((uintptr_t)m.residual % 16 || b.d_model % 4)) return false;
+    const int pieces = m.top_k * a.ppr + a.pps + (m.residual ? 1 : 0);
+    a.ci = (pieces + 63) / 64;
+    a.image = pieces * 16;
+    const int floats = m.top_k * b.d_ff + (has_shared ? m.d_ff_shared : 0);
+    const int chunks = (floats / 4 + 63) / 64;
+    a.ch = (chunks + D2_WAVES - 1) / D2_WAVES;
+    if (a.ci > DOWN2_CI || a.ch > DOWN2_CH) return false;
+    a.hbytes = chunks * 1024;
+    if (a.hbytes + D2_WAVES * 768 + 1024 + D2_WAVES * 2 * a.image > D2_LDS) return false;
+    a.down = (const uint8_t*)b.down;
+    a.down_stride = b.down_stride;
+    a.shared_down = (const uint8_t*)m.shared_down_w;
+    a.h = w.h;
+    a.hs = w.hs;
+    a.sorted_ids = w.sorted_ids;
+    a.sorted_w = w.sorted_w;
+    a.sig = w.sig;
+    a.out = m.out;
+    a.residual = m.residual;
+    a.odt = m.out_dtype;
+    a.k = m.top_k;
+    a.d = b.d_model;
+    a.f = b.d_ff;
+    a.fsh = has_shared ? m.d_ff_shared : 0;
+    a.lpe = lpe;
+    if (out) *out = a;
+    return true;
+}
+
+template <int FMT>
+static int down2_launch_as(const Down2Args& a, int tokens, hipStream_t s) {
+    static bool configured = false;   // (benign if two threads both set it)
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)down2_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, D2_LDS) != hipSuccess)
+            return fail(QMOE_ELAUNCH, "MoE decode (down): cannot reserve %d bytes of LDS", D2_LDS);
+        configured = true;
+    }
+    const int per_wg = D2_WAVES * a.rows;
+    hipLaunchKernelGGL(down2_kernel<FMT>, dim3((a.d + per_wg - 1) / per_wg, tokens), dim3(D2_THREADS), D2_LDS, s, a);
+    return check_launch("qmoe_moe_forward(down)");
+}
+
+bool decode2_down_supported(const qmoe_moe_args& m, const DecodeBuffers& w) { return down2_plan(m, w, stream_grid() / 2, nullptr); }
+
+int decode2_down_launch(const qmoe_moe_args& m, const DecodeBuffers& w, hipStream_t s) {
+    Down2Args a;
+    if (!down2_plan(m, w, stream_grid() / 2, &a)) return fail(QMOE_EUNSUPPORTED, "MoE decode (down): shape not taken");
+    switch (m.bank.down_fmt) {
+    case QMOE_FMT_Q8_0: return down2_launch_as<QMOE_FMT_Q8_0>(a, m.tokens, s);
+    case QMOE_FMT_Q6_K: return down2_launch_as<QMOE_FMT_Q6_K>(a, m.tokens, s);
+    case QMOE_FMT_Q5_K: return down2_launch_as<QMOE_FMT_Q5_K>(a, m.tokens, s);
+    default: return down2_launch_as<QMOE_FMT_Q4_K>(a, m.tokens, s);
+    }
+}
+
+
+
+static bool pairs2_plan(const qmoe_moe_args& m, int waves, Pairs2Shape* out) {
+    const qmoe_expert_bank& b = m.bank;
+    const bool has_shared = m.shared_gate_w != nullptr;
+    if (m.tokens < 1 || m.tokens > PAIRS2_MAX_TOKENS || m.top_k > PAIRS2_MAX_K) return false;
+    if (!span_format(b.gate_fmt) || b.up_fmt != b.gate_fmt) return false;
+    if (has_shared && (m.shared_gate_fmt != b.gate_fmt || m.shared_up_fmt != b.gate_fmt)) return false;
+    if (m.logits && b.n_experts > PAIRS2_MAX_EXPERTS) return false;
+    if (b.d_model % 256 || b.d_model > 2048) return false;
+    const int align = b.gate_fmt == QMOE_FMT_Q6_K ? 2 : 16;
+    const void* bases[4] = {b.gate, b.up, m.shared_gate_w, m.shared_up_w};
+    for (int i = 0; i < (has_shared ? 4 : 2); ++i)
+        if ((uintptr_t)bases[i] % align) return false;
+    if (b.gate_stride % align || b.up_stride % align) return false;
+    if (!x_fast(m.hidden, m.hidden_dtype, b.d_model)) return false;
+    Pairs2Shape x{};
+    x.lr = lanes_per_row(b.d_model);
+    x.ri = 32 / x.lr;
+    if (b.d_ff % x.ri || (has_shared && m.d_ff_shared % x.ri)) return false;
+    x.row_image = (b.d_model >> 8) * pieces_per_256(b.gate_fmt) * 16;
+    x.pph = x.ri * (b.d_model >> 8) * pieces_per_256(b.gate_fmt);
+    x.ipe = b.d_ff / x.ri;
+    x.ish = has_shared ? m.d_ff_shared / x.ri : 0;
+    const long total = (long)x.ish + (long)m.tokens * m.top_k * x.ipe;
+    // quotients by mulhi are exact while dividend x divisor stays below 2^32
+    if ((uint64_t)(total + 3L * waves) * (uint64_t)(x.ipe > m.top_k ? x.ipe : m.top_k) >= (1ull << 32)) return false;
+    x.total = (int)total;
+    x.ipe_magic = magic_of(x.ipe);
+    x.k_magic = magic_of(m.top_k);
+    x.xs_bytes = m.tokens * b.d_model * 4;
+    x.gw = m.tokens == 1 ? 8 : m.tokens == 2 ? 4 : 2;
+    x.nv = (b.n_experts + 64 * x.gw - 1) / (64 * x.gw);
+    if (m.logits && x.nv > PAIRS2_NV) return false;
+    if (m.tokens * (b.d_model >> 8) > 4 * D2_WAVES) return false;   // a wave's 16-bit chunks fit its third ring slot
+    if (out) *out = x;
+    return true;
+}
+
+template <int FMT>
+static int pairs2_launch_as(const DecodeRouteArgs& r, const Pairs2Shape& x, int grid, hipStream_t s) {
+    static bool configured = false;   // (benign if two threads both set it)
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)pairs2_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, D2_LDS) != hipSuccess)
+            return fail(QMOE_ELAUNCH, "MoE decode (gate/up): cannot reserve %d bytes of LDS", D2_LDS);
+        configured = true;
+    }
+    static_assert(PAIRS2_MAX_TOKENS * 2048 * 4 + PAIRS2_MAX_TOKENS * 32 * 8 + PAIRS2_MAX_TOKENS * sizeof(RouteShare) + 1024 +
+                  D2_WAVES * (PAIRS2_PD + 1) * Pairs2Slot<FMT>::BYTES <= D2_LDS, "LDS layout of the gate/up kernel");
+    hipLaunchKernelGGL(pairs2_kernel<FMT>, dim3(grid), dim3(D2_THREADS), D2_LDS, s, r, x);
+    return check_launch("qmoe_moe_forward(route + gate/up)");
+}
+
+bool decode2_pairs_supported(const qmoe_moe_args& m) { return pairs2_plan(m, (stream_grid() / 2) * D2_WAVES, nullptr); }
+
+int decode2_pairs_launch(const qmoe_moe_args& m, const DecodeRouteArgs& r, hipStream_t s) {
+    const int grid = stream_grid() / 2;
+    Pairs2Shape x;
+    if (!pairs2_plan(m, grid * D2_WAVES, &x)) return fail(QMOE_EUNSUPPORTED, "MoE decode (gate/up): shape not taken");
+    switch (m.bank.gate_fmt) {
+    case QMOE_FMT_Q8_0: return pairs2_launch_as<QMOE_FMT_Q8_0>(r, x, grid, s);
+    case QMOE_FMT_Q6_K: return pairs2_launch_as<QMOE_FMT_Q6_K>(r, x, grid, s);
+    case QMOE_FMT_Q5_K: return pairs2_launch_as<QMOE_FMT_Q5_K>(r, x, grid, s);
+    default: return pairs2_launch_as<QMOE_FMT_Q4_K>(r, x, grid, s);
+    }
+}
+
+}  // namespace qmoe
+
+#ifdef QMOE_TIMELINE
+// Copies the stamps of both kernels to `out` (2 x 4096 x 8 unsigned 64-bit values) after the device is idle.
+extern "C" int qmoe_timeline_read(unsigned long long* out) {
+    if (hipDeviceSynchronize() != hipSuccess) return QMOE_ELAUNCH;
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(qmoe::timeline), sizeof(qmoe::timeline)) == hipSuccess ? QMOE_OK : QMOE_ELAUNCH;
+}
+#endif

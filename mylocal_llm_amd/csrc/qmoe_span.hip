@@ -20,15 +20,6 @@ namespace qmoe {
 #define QMOE_LDS __attribute__((address_space(3)))
 typedef QMOE_LDS uint32_t* lds_counter;
 
-// Activations in LDS as fp32: 16-byte granules XOR-swizzled inside groups of 16 64-element units,
-// so that lanes reading granule i of consecutive units hit different banks without padding.
-// The map is its own inverse.
-__device__ __forceinline__ int swizzled_granule(int g) { return (g & ~15) | ((g & 15) ^ ((g >> 4) & 15)); }
-struct SwizzledX {
-    const uint8_t* xs;
-    __device__ __forceinline__ float4 operator()(int col) const { return *(const float4*)(xs + 16 * swizzled_granule(col >> 2)); }
-};
-
 // Rows of one work item and 4096-column parts of a row.
 __host__ __device__ inline int span_parts(int k) { return ((k >> 6) + 63) >> 6; }
 __host__ __device__ inline int span_rows_per_item(int k) { return (k >> 6) <= 64 ? 64 / lanes_per_row(k) : 1; }

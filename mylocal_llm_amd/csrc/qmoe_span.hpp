@@ -42,6 +42,15 @@ __device__ __forceinline__ void dma16_masked(const void* base, uint32_t voff, ui
                  : "=&s"(save) : "v"(voff), "s"(uniform((const uint8_t*)base)), "s"(mask) : "memory");
 }
 
+// Activations in LDS as fp32: 16-byte granules XOR-swizzled inside groups of 16 64-element units,
+// so that lanes reading granule i of consecutive units hit different banks without padding.
+// The map is its own inverse.
+__device__ __forceinline__ int swizzled_granule(int g) { return (g & ~15) | ((g & 15) ^ ((g >> 4) & 15)); }
+struct SwizzledX {
+    const uint8_t* xs;
+    __device__ __forceinline__ float4 operator()(int col) const { return *(const float4*)(xs + 16 * swizzled_granule(col >> 2)); }
+};
+
 template <int FMT> struct SpanFmt;
 
 template <> struct SpanFmt<QMOE_FMT_Q8_0> {
