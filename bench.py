@@ -217,7 +217,7 @@ def cpu_baseline(budget_s=24.0):
 
 
 TIMELINE_STAMPS = {
-    0: ("route + gate/up kernel", ["wave enters", "token routed / activations staged", "",
+    0: ("route + gate/up kernel", ["wave enters", "row selected / summed, activations staged", "",
                                    "at the barrier", "past the barrier", "first item's rows arrived", "wave ends"]),
     1: ("down kernel", ["wave enters", "routing arrived, two rows requested", "activations arrived", "past the barrier",
                         "first row arrived", "wave ends", "(routing arrived)", "(row addresses ready)"]),

@@ -474,7 +474,7 @@ int decode_launch(const qmoe_moe_args& a, const DecodeBuffers& w, hipStream_t s)
     int rc;
     const bool fused = a.tokens <= FUSED_MAX_TOKENS && a.top_k + 1 <= FUSED_MAX_SLOTS && b.d_model <= 4096 &&
                        (!a.logits || b.n_experts <= FUSED_MAX_EXPERTS);
-    if (a.tokens <= FUSED_MAX_TOKENS && decode2_pairs_supported(a)) {
+    if (decode2_pairs_supported(a)) {
         if ((rc = decode2_pairs_launch(a, r, s))) return rc;
     } else if (fused) {
         r.shared_apart = has_shared;   // streamed once for all tokens, beside the routing

@@ -299,11 +299,11 @@ __global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a)
 // ================================================================================================
 // routing + gate/up
 // ================================================================================================
-static constexpr int PAIRS2_MAX_TOKENS = 4;
-static constexpr int PAIRS2_MAX_EXPERTS = 1024;   // two router values per lane at most when eight waves share a row
+static constexpr int PAIRS2_MAX_TOKENS = 4;         // tokens a workgroup routes and holds activations of
+static constexpr int PAIRS2_MAX_STEP_TOKENS = 16;   // tokens of a launch: groups of up to four
+static constexpr int PAIRS2_MAX_EXPERTS = 1024;   // a router row of 4 KB fits the ring slots it is staged in
 static constexpr int PAIRS2_MAX_K = 16;
 static constexpr int PAIRS2_PD = 2;               // slots requested ahead of the one being multiplied
-static constexpr int PAIRS2_NV = 8;               // most router values per lane
 
 struct Pairs2Shape {
     int lr;            // lanes per row (8, 16 or 32)
@@ -313,41 +313,29 @@ struct Pairs2Shape {
     int ipe, ish;      // items per expert pair (f / ri), of the shared pair (fsh / ri)
     int total;         // ish + tokens * k * ipe
     uint32_t ipe_magic, k_magic;   // floor(2^32 / d) + 1: exact quotients by mulhi for the sizes taken here
-    int xs_bytes;      // LDS bytes of the staged activations (tokens * d * 4)
-    int gw;            // waves that route one token together: 8, 4 or 2
-    int nv;            // router values per lane: ceil(n_experts / (64 gw))
+    int xs_bytes;      // LDS bytes of the staged activations (tokens of a group * d * 4)
+    int groups;        // token groups of the launch: ceil(tokens / 4)
+    int group_tokens;  // tokens per group (the last group may have fewer)
+    int nv;            // router values per lane: 8 (up to 512 experts) or 16
 };
 
-// What the waves that route one token together leave for each other in LDS.
+// What the two waves that route a token leave in LDS: the row's maximum and softmax denominator.
 struct RouteShare {
-    uint32_t max_key[D2_WAVES];
-    uint32_t has_nan[D2_WAVES];
-    double partial[D2_WAVES];
-    uint32_t cand_key[D2_WAVES * PAIRS2_MAX_K];   // each wave's own best k, best first
-    int cand_id[D2_WAVES * PAIRS2_MAX_K];
+    float m, denom;
 };
 
-// The best k of one wave's stretch of a router row (NV values per lane, value j of a lane is expert
-// id0 + lane + 64 j): lane s < k receives the s-th best as (order key, expert id); the stretch's best
-// key and whether it holds a NaN come back for the row's maximum.  Keys: order_key with every NaN
-// raised to 1 (below -inf, above 0 = "taken or absent"); ties go to the lower id.
+// A router row in LDS (value i at byte 4 i), NV values per lane (value j of a lane is expert
+// lane + 64 j).  Keys: order_key with every NaN raised to 1 (below -inf, above 0 = "taken or
+// absent"); a round is one DPP maximum of the lanes' best keys; ties go to the lower id.
 template <int NV>
-__device__ __forceinline__ void stretch_best(const float* v, int id0, int n, int k, uint32_t& wave_best, bool& any_nan,
-                                             uint32_t& my_key, int& my_id) {
+__device__ __forceinline__ void row_select(const uint8_t* row, int n, int k, uint32_t& my_key, int& my_id) {
     const int lane = threadIdx.x & 63;
     uint32_t key[NV];
-    uint32_t best = 0u;
-    bool nan_seen = false;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-        const bool valid = id0 + lane + 64 * j < n;
-        const uint32_t ok = order_key(v[j]);
-        key[j] = valid ? (ok ? ok : 1u) : 0u;
-        nan_seen |= valid && ok == 0u;
-        best = key[j] > best ? key[j] : best;
+        const uint32_t ok = order_key(*(const float*)(row + 256 * j + 4 * lane));
+        key[j] = lane + 64 * j < n ? (ok ? ok : 1u) : 0u;
     }
-    wave_best = wave_max_u32(best);
-    any_nan = __any(nan_seen);
     for (int slot = 0; slot < k; ++slot) {
         uint32_t c = 0u;
 #pragma unroll
@@ -364,8 +352,32 @@ __device__ __forceinline__ void stretch_best(const float* v, int id0, int n, int
 #pragma unroll
         for (int j = 0; j < NV; ++j)
             if (j == wj) key[j] = lane == wl ? 0u : key[j];
-        if (lane == slot) { my_key = win; my_id = id0 + wl + 64 * wj; }
+        if (lane == slot) { my_key = win; my_id = wl + 64 * wj; }
     }
+}
+// The row's maximum (NaN if the row holds one, as the portable graph computes it) and the softmax
+// denominator sum exp(v - max), accumulated in double.
+template <int NV>
+__device__ __forceinline__ void row_softmax_sum(const uint8_t* row, int n, float& m, float& denom) {
+    const int lane = threadIdx.x & 63;
+    float v[NV];
+    uint32_t best = 0u;
+    bool nan_seen = false;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        v[j] = *(const float*)(row + 256 * j + 4 * lane);
+        const bool valid = lane + 64 * j < n;
+        const uint32_t ok = order_key(v[j]);
+        const uint32_t key = valid ? (ok ? ok : 1u) : 0u;
+        nan_seen |= valid && ok == 0u;
+        best = key > best ? key : best;
+    }
+    m = __any(nan_seen) ? __uint_as_float(0x7FC00000u) : key_value(wave_max_u32(best));
+    double part = 0.0;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+        if (lane + 64 * j < n) part += (double)expf(v[j] - m);
+    denom = (float)wave_sum_f64(part);
 }
 
 template <int FMT> struct Pairs2Slot {
@@ -375,13 +387,36 @@ template <int FMT> struct Pairs2Slot {
 
 // LDS: [activations fp32, swizzled | sorted ids per token | dump | rings: 8 waves x 3 slots]
 template <int FMT>
-__global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRouteArgs a, const Pairs2Shape x) {
+__global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRouteArgs step, const Pairs2Shape shape) {
     using U = Unit64<FMT>;
     using S = SpanFmt<FMT>;
     using SL = Pairs2Slot<FMT>;
     constexpr int PD = PAIRS2_PD, NS = PD + 1, CH = SL::CH;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63, wave = uniform((int)(threadIdx.x >> 6));
+    // More than four tokens are cut into groups of up to four; the workgroups are dealt out to the
+    // groups in turn, and each group is a step of its own on its share of the chip: `a`, `x`, `wg` and
+    // `wgs` below are that step (its tokens, its outputs, this workgroup's place in it).
+    DecodeRouteArgs a = step;
+    Pairs2Shape x = shape;
+    const int wg_index = blockIdx.x / shape.groups, wgs = (gridDim.x - blockIdx.x % shape.groups + shape.groups - 1) / shape.groups;
+    {
+        const int q = blockIdx.x % shape.groups, token0 = q * shape.group_tokens;
+        const int mine = step.tokens - token0 < shape.group_tokens ? step.tokens - token0 : shape.group_tokens;
+        a.tokens = mine;
+        a.hidden = (const uint8_t*)step.hidden + (size_t)token0 * step.d * (step.xdt == QMOE_DT_F32 ? 4 : 2);
+        if (step.logits) a.logits = step.logits + (size_t)token0 * step.n_experts;
+        if (step.in_ids) a.in_ids = step.in_ids + (size_t)token0 * step.k;
+        if (step.in_weights) a.in_weights = step.in_weights + (size_t)token0 * step.k;
+        if (step.out_weights) a.out_weights = step.out_weights + (size_t)token0 * step.k;
+        if (step.out_ids) a.out_ids = step.out_ids + (size_t)token0 * step.k;
+        a.sorted_ids = step.sorted_ids + (size_t)token0 * step.k;
+        a.sorted_w = step.sorted_w + (size_t)token0 * step.k;
+        a.sig = step.sig + token0;
+        a.h = step.h + (size_t)token0 * step.k * step.f;
+        a.hs = step.hs + (size_t)token0 * step.fsh;
+        x.total = x.ish + mine * step.k * x.ipe;
+    }
     const int T = a.tokens, k = a.k;
     uint8_t* const xs = lds;
     int64_t* const sid = (int64_t*)(lds + x.xs_bytes);                  // [PAIRS2_MAX_TOKENS][32]
@@ -474,43 +509,40 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
     };
 
     // ---- routing, activations, and a first row pair of the shared expert ---------------------------
-    // The waves of a workgroup route together: `gw` waves per token, each with its own stretch of
-    // the router row (one value per lane for 512 experts and one token).  A wave picks the best k of
-    // its stretch, the waves of a token exchange those through LDS, and each of them then picks the
-    // best k of the gw * k candidates by itself -- the same order keys, the same tie rule (lower id),
-    // so the result is the single-wave router's, in a fraction of its instructions.  Every load of
-    // this part is an inline-assembly load with a wait of its own: the row pair of the shared expert
-    // that a wave requests first must not be waited for by anything here.
+    // Two waves route a token, side by side: wave 2 t picks the k best of the row (ten serial rounds
+    // of a wave-wide maximum: the long pole), wave 2 t + 1 meanwhile finds the row's maximum and the
+    // softmax denominator.  All waves stage the tokens' activations and request a first row pair
+    // of the shared expert, which needs no routing.  Everything fetched here travels by DMA into
+    // LDS (router rows and 16-bit activations into the wave's own ring slots, which are free until
+    // the barrier; fp32 activations straight to their place): no register waits for a load, and the
+    // row pair on its way is waited for by nothing.
     QMOE_STAMP(0, 0);
     const int n = a.n_experts;
-    const int group = wave / x.gw, wg = wave - group * x.gw;   // token `group`, position in its group
-    const bool routes = group < T;
+    const int token = wave >> 1;                     // the token this wave helps to route, if < T
+    const bool routes = token < T, selects = routes && !(wave & 1);
     const bool from_logits = a.logits != nullptr;
-    RouteShare* const share = (RouteShare*)(sid + PAIRS2_MAX_TOKENS * 32) + group;
-    // The waves that publish the routing (workgroup 0, the first wave of each token's group) take
-    // no items: they have the admission gate to compute, with ordinary loads, which must not meet
-    // requests in flight.  All other waves share the item stream.
-    const bool publishes = blockIdx.x == 0 && routes && wg == 0;
+    RouteShare* const share = (RouteShare*)(sid + PAIRS2_MAX_TOKENS * 32) + token;
+    // The waves that publish the routing (the selecting waves of workgroup 0) take no items: they
+    // have the admission gate to compute, with ordinary loads, which must not meet requests in
+    // flight.  All other waves share the item stream.
+    const bool publishes = wg_index == 0 && selects;
     // (a) the routing given by the caller (ordinary loads, waited for before anything else is issued)
     float weight = 0.f;
     int64_t id = 0;
-    if (routes && !from_logits) {
+    if (selects && !from_logits) {
         const int kk = lane < k ? lane : k - 1;
-        id = a.in_ids[(size_t)group * k + kk];
-        weight = a.in_weights[(size_t)group * k + kk];
+        id = a.in_ids[(size_t)token * k + kk];
+        weight = a.in_weights[(size_t)token * k + kk];
         asm volatile("" ::"v"((uint32_t)id), "v"((uint32_t)((uint64_t)id >> 32)), "v"(weight) : "memory");
     }
-    // ... or the wave's stretch of the router row.  Everything a wave fetches here goes to LDS by
-    // DMA (router values and 16-bit activations into the wave's own ring slots, which are free until
-    // the barrier; fp32 activations straight to their place), so that no register waits for a load.
-    const int id0 = wg * 64 * x.nv;   // first expert of this wave's stretch
-    uint8_t* const lds_logits = ring + SL::BYTES;       // value j of lane l at 256 j + 4 l
-    uint8_t* const lds_xraw = ring + 2 * SL::BYTES;     // this wave's 16-bit chunks, 512 bytes each
+    // ... or the router row, into the second slot of this wave's ring (and on into the third)
+    uint8_t* const lds_logits = ring + SL::BYTES;              // value i at byte 4 i, up to 4 KB
+    uint8_t* const lds_xraw = ring + NS * SL::BYTES - 2048;    // this wave's 16-bit chunks, 512 bytes each
     int n_loads = 0;
     if (routes && from_logits) {
-        const float* const row = a.logits + (size_t)group * n;
+        const float* const row = a.logits + (size_t)token * n;
         for (int j = 0; j < x.nv; ++j) {
-            const int at = id0 + lane + 64 * j;
+            const int at = lane + 64 * j;
             set_m0((uint32_t)(uintptr_t)(lds_logits + 256 * j));
             dma4_at(row + (at < n ? at : n - 1));
             ++n_loads;
@@ -537,11 +569,11 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
             ++n_loads;
         }
     }
-    n_loads -= n_logit_loads;   // (requests newer than the router values)
+    n_loads -= n_logit_loads;   // (requests newer than the router row)
     // (c) a row pair of the shared expert, if the wave's first item is one
-    const int W = gridDim.x * D2_WAVES - T;                      // waves that take items
-    const int before = (wave + x.gw - 1) / x.gw;   // publishing waves of workgroup 0 ahead of this one
-    const int me = blockIdx.x * D2_WAVES + wave - (blockIdx.x == 0 ? (before < T ? before : T) : T);
+    const int W = wgs * D2_WAVES - T;                             // waves of this group that take items
+    const int before = (wave + 1) >> 1;                           // publishing waves of the group's first workgroup ahead of this one
+    const int me = wg_index * D2_WAVES + wave - (wg_index == 0 ? (before < T ? before : T) : T);
     const int g0 = publishes ? x.total : me;                      // this wave's items are g0, g0 + W, ...
     const bool early = g0 < x.ish;   // the first item is a shared one, requested before the routing is known
     Item it[NS];
@@ -550,52 +582,25 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
         request(0, it[0]);
         n_loads += CH;
     }
-    // (d) the wave's own best k
+    // (d) the row's k best on one wave, its maximum and denominator on the other
     wait_vmcnt_rt(n_loads);
-    uint32_t my_key = 0u;
-    int my_id = 0;
-    float m = 0.f, denom = 1.f;
-    float v[PAIRS2_NV];
-#pragma unroll
-    for (int j = 0; j < PAIRS2_NV; ++j) v[j] = j < x.nv ? *(const float*)(lds_logits + 256 * j + 4 * lane) : 0.f;
+    uint32_t sel_key = 0u;
+    int sel_id = 0;
     if (routes && from_logits) {
-        uint32_t wave_best = 0u;
-        bool any_nan = false;
-        switch (x.nv) {
-        case 1: stretch_best<1>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
-        case 2: stretch_best<2>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
-        case 4: stretch_best<4>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
-        default: stretch_best<8>(v, id0, n, k, wave_best, any_nan, my_key, my_id); break;
+        if (selects) {
+            if (x.nv <= 8) row_select<8>(lds_logits, n, k, sel_key, sel_id);
+            else row_select<16>(lds_logits, n, k, sel_key, sel_id);
+        } else {
+            float m, denom;
+            if (x.nv <= 8) row_softmax_sum<8>(lds_logits, n, m, denom);
+            else row_softmax_sum<16>(lds_logits, n, m, denom);
+            if (lane == 0) {
+                share->m = m;
+                share->denom = denom;
+            }
         }
-        if (lane == 0) {
-            share->max_key[wg] = wave_best;
-            share->has_nan[wg] = any_nan ? 1u : 0u;
-        }
-        if (lane < k) {
-            share->cand_key[wg * k + lane] = my_key;
-            share->cand_id[wg * k + lane] = my_id;
-        }
-        QMOE_STAMP(0, 1);
-        __syncthreads();
-        // (e) the row's maximum, then this stretch's part of the softmax denominator
-        uint32_t row_best = 0u, row_nan = 0u;
-        for (int w2 = 0; w2 < x.gw; ++w2) {
-            const uint32_t o = share->max_key[w2];
-            row_best = o > row_best ? o : row_best;
-            row_nan |= share->has_nan[w2];
-        }
-        m = row_nan ? __uint_as_float(0x7FC00000u) : key_value(row_best);   // maximum with NaN propagation
-        double part = 0.0;
-#pragma unroll
-        for (int j = 0; j < PAIRS2_NV; ++j)
-            if (j < x.nv && id0 + lane + 64 * j < n) part += (double)expf(v[j] - m);
-        part = wave_sum_f64(part);
-        if (lane == 0) share->partial[wg] = part;
-    } else {
-        QMOE_STAMP(0, 1);
-        __syncthreads();
     }
-    // (f) activations into LDS as fp32 (they have long arrived; only the row pair may still travel)
+    // (e) activations into LDS as fp32 (they have long arrived; only the row pair may still travel)
     wait_vmcnt_rt(early ? CH : 0);
     if (a.xdt != QMOE_DT_F32) {
         for (int i = 0; wave + D2_WAVES * i < chunks; ++i) {
@@ -613,38 +618,21 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
             *(float4*)(xs + (size_t)t * a.d * 4 + 16 * swizzled_granule(gran)) = f;
         }
     }
+    QMOE_STAMP(0, 1);
     __syncthreads();
-    // (g) every wave of a token's group picks the best k of the group's candidates by itself
-    if (routes && from_logits) {
-        double total = 0.0;
-        for (int w2 = 0; w2 < x.gw; ++w2) total += share->partial[w2];
-        denom = (float)total;
-        const int cands = x.gw * k;   // candidate i = wave i / k, its rank i % k: ties fall to the lower id as before
-        uint32_t ck[2];
-#pragma unroll
-        for (int j = 0; j < 2; ++j) ck[j] = lane + 64 * j < cands ? share->cand_key[lane + 64 * j] : 0u;
-        uint32_t sel_key = 0u;
-        int sel_at = 0;
-        for (int slot = 0; slot < k; ++slot) {
-            const uint32_t c = ck[0] > ck[1] ? ck[0] : ck[1];
-            const uint32_t win = wave_max_u32(c);
-            const unsigned long long b0 = __ballot(ck[0] == win), b1 = __ballot(ck[1] == win);
-            const int wj = b0 ? 0 : 1;
-            const int wl = __builtin_ctzll(b0 ? b0 : b1);
-            if (wj == 0) ck[0] = lane == wl ? 0u : ck[0];
-            else ck[1] = lane == wl ? 0u : ck[1];
-            if (lane == slot) { sel_key = win; sel_at = wl + 64 * wj; }
+    // (f) the selecting wave: probabilities, renormalisation, the selections sorted by expert id
+    if (selects) {
+        if (from_logits) {
+            const float m = share->m, denom = share->denom;
+            id = sel_id;
+            // probabilities in parallel; their sum in selection order
+            const float p = lane < k ? expf(key_value(sel_key) - m) / denom : 0.0f;
+            float mass = 0.0f;
+            for (int slot = 0; slot < k; ++slot) mass += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), slot));
+            float norm = 1.0f;
+            if (a.renorm) norm = isnan(mass) ? mass : fmaxf(mass, a.floor_value);
+            weight = a.renorm ? p / norm : p;
         }
-        id = lane < k ? share->cand_id[sel_at] : 0;
-        // probabilities in parallel; their sum in selection order
-        const float p = lane < k ? expf(key_value(sel_key) - m) / denom : 0.0f;
-        float mass = 0.0f;
-        for (int slot = 0; slot < k; ++slot) mass += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), slot));
-        float norm = 1.0f;
-        if (a.renorm) norm = isnan(mass) ? mass : fmaxf(mass, a.floor_value);
-        weight = a.renorm ? p / norm : p;
-    }
-    if (routes) {
         // rank of a selection in ascending expert id; equal ids keep slot order.  An id outside the
         // bank, or an expert the token has named in an earlier slot already, contributes nothing.
         int rank = 0;
@@ -656,15 +644,15 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
         }
         if (lane < k) {
             const bool in_range = id >= 0 && id < n, ok = in_range && !again;
-            sid[group * 32 + rank] = ok ? id : -1;   // (every wave of the group writes the same values)
-            if (publishes) {        // one wave publishes the routing for the down kernel and the caller
+            sid[token * 32 + rank] = ok ? id : -1;
+            if (publishes) {   // for the down kernel and the caller
                 if (!ok && a.status_out) atomicOr(a.status_out, (in_range ? 0 : 1) | (again ? 2 : 0));
                 if (a.out_weights) {
-                    a.out_weights[(size_t)group * k + lane] = weight;
-                    a.out_ids[(size_t)group * k + lane] = id;
+                    a.out_weights[(size_t)token * k + lane] = weight;
+                    a.out_ids[(size_t)token * k + lane] = id;
                 }
-                a.sorted_ids[(size_t)group * k + rank] = ok ? (int)id : -1;
-                a.sorted_w[(size_t)group * k + rank] = weight;
+                a.sorted_ids[(size_t)token * k + rank] = ok ? (int)id : -1;
+                a.sorted_w[(size_t)token * k + rank] = weight;
             }
         }
     }
@@ -677,14 +665,14 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
         float adm = 0.f;
         if (a.shared_gate) {
             for (int c = lane; c < (a.d >> 2); c += 64) {
-                const float4 h = *(const float4*)(xs + (size_t)group * a.d * 4 + 16 * swizzled_granule(c));
+                const float4 h = *(const float4*)(xs + (size_t)token * a.d * 4 + 16 * swizzled_granule(c));
                 const float4 gv = ldg<float4>(a.shared_gate + 4 * c);
                 adm += (h.x * gv.x + h.y * gv.y) + (h.z * gv.z + h.w * gv.w);
             }
             adm = wave_sum(adm);
         }
         // sigmoid(hidden . g) without overflow
-        if (lane == 0) a.sig[group] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
+        if (lane == 0) a.sig[token] = a.shared_gate ? (adm >= 0.f ? 1.f / (1.f + expf(-adm)) : expf(adm) / (1.f + expf(adm))) : 1.f;
         return;
     }
 
@@ -809,7 +797,7 @@ int decode2_down_launch(const qmoe_moe_args& m, const DecodeBuffers& w, hipStrea
 static bool pairs2_plan(const qmoe_moe_args& m, int waves, Pairs2Shape* out) {
     const qmoe_expert_bank& b = m.bank;
     const bool has_shared = m.shared_gate_w != nullptr;
-    if (m.tokens < 1 || m.tokens > PAIRS2_MAX_TOKENS || m.top_k > PAIRS2_MAX_K) return false;
+    if (m.tokens < 1 || m.tokens > PAIRS2_MAX_STEP_TOKENS || m.top_k > PAIRS2_MAX_K) return false;
     if (!span_format(b.gate_fmt) || b.up_fmt != b.gate_fmt) return false;
     if (has_shared && (m.shared_gate_fmt != b.gate_fmt || m.shared_up_fmt != b.gate_fmt)) return false;
     if (m.logits && b.n_experts > PAIRS2_MAX_EXPERTS) return false;
@@ -828,17 +816,18 @@ static bool pairs2_plan(const qmoe_moe_args& m, int waves, Pairs2Shape* out) {
     x.pph = x.ri * (b.d_model >> 8) * pieces_per_256(b.gate_fmt);
     x.ipe = b.d_ff / x.ri;
     x.ish = has_shared ? m.d_ff_shared / x.ri : 0;
-    const long total = (long)x.ish + (long)m.tokens * m.top_k * x.ipe;
+    x.groups = (m.tokens + PAIRS2_MAX_TOKENS - 1) / PAIRS2_MAX_TOKENS;
+    x.group_tokens = (m.tokens + x.groups - 1) / x.groups;
+    if (x.groups * 8 > waves / D2_WAVES) return false;   // (a group wants a few workgroups at least)
+    const long total = (long)x.ish + (long)x.group_tokens * m.top_k * x.ipe;
     // quotients by mulhi are exact while dividend x divisor stays below 2^32
     if ((uint64_t)(total + 3L * waves) * (uint64_t)(x.ipe > m.top_k ? x.ipe : m.top_k) >= (1ull << 32)) return false;
     x.total = (int)total;
     x.ipe_magic = magic_of(x.ipe);
     x.k_magic = magic_of(m.top_k);
-    x.xs_bytes = m.tokens * b.d_model * 4;
-    x.gw = m.tokens == 1 ? 8 : m.tokens == 2 ? 4 : 2;
-    x.nv = (b.n_experts + 64 * x.gw - 1) / (64 * x.gw);
-    if (m.logits && x.nv > PAIRS2_NV) return false;
-    if (m.tokens * (b.d_model >> 8) > 4 * D2_WAVES) return false;   // a wave's 16-bit chunks fit its third ring slot
+    x.xs_bytes = x.group_tokens * b.d_model * 4;
+    x.nv = b.n_experts <= 512 ? 8 : 16;
+    if (x.group_tokens * (b.d_model >> 8) > 4 * D2_WAVES) return false;   // a wave's 16-bit chunks fit the end of its ring
     if (out) *out = x;
     return true;
 }
