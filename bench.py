@@ -218,7 +218,7 @@ def cpu_baseline(budget_s=24.0):
 
 TIMELINE_STAMPS = {
     0: ("route + gate/up kernel", ["wave enters", "row selected / summed, activations staged", "",
-                                   "at the barrier", "past the barrier", "first item's rows arrived", "wave ends"]),
+                                   "at the barrier", "past the barrier", "first item's rows arrived", "wave ends", "(first instruction)"]),
     1: ("down kernel", ["wave enters", "routing arrived, two rows requested", "activations arrived", "past the barrier",
                         "first row arrived", "wave ends", "(routing arrived)", "(row addresses ready)"]),
 }

@@ -56,6 +56,12 @@ __device__ __forceinline__ void dma16_at(const uint8_t* lane_address) {
 __device__ __forceinline__ void dma4_at(const void* lane_address) {
     asm volatile("global_load_lds_dword %0, off" ::"v"(lane_address) : "memory");
 }
+__device__ __forceinline__ void dma4_at_masked(const void* lane_address, uint64_t mask) {
+    uint64_t save;
+    mask = ((uint64_t)(uint32_t)uniform((int)(mask >> 32)) << 32) | (uint32_t)uniform((int)(uint32_t)mask);
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %2\n\tglobal_load_lds_dword %1, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(save) : "v"(lane_address), "s"(mask) : "memory");
+}
 // ... on the lanes of `mask` only (a wave-uniform 64-bit lane mask, not zero)
 __device__ __forceinline__ void dma16_at_masked(const uint8_t* lane_address, uint64_t mask) {
     uint64_t save;
@@ -151,10 +157,8 @@ __global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a)
     const int lane = threadIdx.x & 63, wave = uniform((int)(threadIdx.x >> 6));
     const int k = a.k, R = a.rows, t = blockIdx.y;
     uint8_t* const hbuf = lds;
-    int* const tab_ids = (int*)(lds + a.hbytes + wave * 768);   // this wave's copy of the token's routing: 64 ids,
-    float* const tab_w = (float*)(tab_ids + 64);                 // 64 weights, the sigmoid gate (entries past k repeat entry k - 1)
-    float* const tab_sig = tab_w + 64;
-    uint8_t* const dump = lds + a.hbytes + D2_WAVES * 768;
+    int* const tab_ids = (int*)(lds + a.hbytes + wave * 256);   // this wave's copy of the token's routing: 16 ids, 16 weights, the gate
+    uint8_t* const dump = lds + a.hbytes + D2_WAVES * 256;
     uint8_t* const ring = dump + 1024 + wave * (2 * a.image);
     const int row0 = (blockIdx.x * D2_WAVES + wave) * R;   // first output row of this wave
     const int64_t rb_r = row_bytes_dev(FMT, a.f), rb_s = row_bytes_dev(FMT, a.fsh);
@@ -162,13 +166,15 @@ __global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a)
     QMOE_STAMP(1, 0);
 
     // ---- 1. the token's routing, by DMA into this wave's table (no register waits for a load) ------
-    const int kk = lane < k ? lane : k - 1;
-    set_m0((uint32_t)(uintptr_t)tab_ids);
-    dma4_at(a.sorted_ids + t * k + kk);
-    set_m0((uint32_t)(uintptr_t)tab_w);
-    dma4_at(a.sorted_w + t * k + kk);
-    set_m0((uint32_t)(uintptr_t)tab_sig);
-    dma4_at(a.sig + t);
+    // one request: lanes 0..15 fetch the expert ids (entries past k repeat entry k - 1), lanes
+    // 16..31 the weights, the rest the sigmoid gate
+    {
+        const int kk = (lane & 15) < k ? (lane & 15) : k - 1;
+        const void* const from = lane < 16 ? (const void*)(a.sorted_ids + t * k + kk)
+                               : lane < 32 ? (const void*)(a.sorted_w + t * k + kk) : (const void*)(a.sig + t);
+        set_m0((uint32_t)(uintptr_t)tab_ids);
+        dma4_at(from);
+    }
 
     // ---- 2. the token's activations: [h of its k slots | hs], swizzled while they travel --------
     // LDS granule P = 64 chunk + lane receives source granule swizzled(P); a wave brings chunks
@@ -190,52 +196,63 @@ __global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a)
             }
     }
 
-    // ---- 3. the routing into registers and LDS ----------------------------------------------------
-    wait_vmcnt_rt(a.ch);
-    QMOE_STAMP(1, 6);
-    const float route_w = lane < k ? tab_w[lane] : 0.f;   // lane j holds weight j
-    const float sg = tab_sig[0];
-
-    // ---- 4. where piece p = lane + 64 c of a row image comes from ---------------------------------
-    // p < k ppr: piece p % ppr of expert slot p / ppr; then the pieces of the shared row.
-    // With a residual, one more piece: the 16 bytes that hold the residual's value of the row (an
-    // ordinary load here would make the compiler wait for everything in flight).
+    // ---- 3. where piece p = lane + 64 c of a row image comes from ---------------------------------
+    // p < k ppr: piece p % ppr of expert slot p / ppr; then the pieces of the shared row.  What does
+    // not depend on the routing is worked out while the routing travels: row 0's address without
+    // the expert's offset, and the bytes between consecutive rows.
     const uint8_t* src[DOWN2_CI];
-    uint32_t is_shared = 0, is_residual = 0;
-    const int routed_pieces = k * a.ppr, weight_pieces = routed_pieces + a.pps, pieces = weight_pieces + (a.residual ? 1 : 0);
+    uint32_t stride[DOWN2_CI];
+    uint32_t slot_of = 0;   // 4 bits per instruction: the expert slot of a routed piece
+    uint32_t is_routed = 0;
+    const int routed_pieces = k * a.ppr, pieces = routed_pieces + a.pps;
 #pragma unroll
     for (int c = 0; c < DOWN2_CI; ++c) {
         const int p = lane + 64 * c;
-        const uint8_t* from = a.down;
+        src[c] = a.down;
+        stride[c] = 0u;
         if (p < routed_pieces) {
             const int j = (int)__umulhi((uint32_t)p, a.ppr_magic), q = p - j * a.ppr;
-            const int e = tab_ids[j];
-            from = a.down + (int64_t)(e >= 0 ? e : 0) * a.down_stride + S::src(q);
-        } else if (p < weight_pieces) {
-            from = a.shared_down + S::src(p - routed_pieces);
-            is_shared |= 1u << c;
+            src[c] = a.down + S::src(q);
+            stride[c] = (uint32_t)rb_r;
+            slot_of |= (uint32_t)j << (4 * c);
+            is_routed |= 1u << c;
         } else if (p < pieces) {
-            from = (const uint8_t*)(a.residual + (size_t)t * a.d);
-            is_residual |= 1u << c;
+            src[c] = a.shared_down + S::src(p - routed_pieces);
+            stride[c] = (uint32_t)rb_s;
         }
-        src[c] = from;
     }
     const int last_lanes = pieces - 64 * (a.ci - 1);   // lanes of the last instruction, 1..64
     const uint64_t last_mask = last_lanes >= 64 ? ~0ull : ((1ull << last_lanes) - 1);
+    wait_vmcnt_rt(a.ch);
+    QMOE_STAMP(1, 6);
+    const float route_w = lane < k ? __int_as_float(tab_ids[16 + lane]) : 0.f;   // lane j holds weight j
+    const float sg = __int_as_float(tab_ids[32]);
+#pragma unroll
+    for (int c = 0; c < DOWN2_CI; ++c)
+        if ((is_routed >> c) & 1u) {
+            const int e = tab_ids[(slot_of >> (4 * c)) & 15u];
+            src[c] += (int64_t)(e >= 0 ? e : 0) * a.down_stride;
+        }
+    // With a residual, its value of the row travels with the row, behind the image (an ordinary
+    // load here would make the compiler wait for everything in flight).
+    const float* const res_row = a.residual ? a.residual + (size_t)t * a.d : nullptr;
     auto request = [&](int i) {   // row i of this wave into slot i & 1
-        const int row = clamp_row(i);
-        const int64_t at_r = (int64_t)row * rb_r, at_s = (int64_t)row * rb_s, at_res = (int64_t)(row & ~3) * 4;
+        const uint32_t row = (uint32_t)clamp_row(i);
         uint8_t* const img = ring + (i & 1) * a.image;
 #pragma unroll
         for (int c = 0; c < DOWN2_CI; ++c)
             if (c < a.ci) {
-                const uint8_t* const from = src[c] + (((is_shared >> c) & 1u) ? at_s : ((is_residual >> c) & 1u) ? at_res : at_r);
+                const uint8_t* const from = src[c] + (uint64_t)row * stride[c];
                 set_m0((uint32_t)(uintptr_t)(img + 1024 * c));
                 if (c + 1 < a.ci) dma16_at(from);
                 else dma16_at_masked(from, last_mask);
             }
+        if (res_row) {
+            set_m0((uint32_t)(uintptr_t)(img + pieces * 16));
+            dma4_at_masked(res_row + row, 1ull);
+        }
     };
-    const int per_request = a.ci;
+    const int per_request = a.ci + (res_row ? 1 : 0);
     QMOE_STAMP(1, 7);
     request(0);
     if (R > 1) request(1);
@@ -270,7 +287,7 @@ __global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a)
         uint32_t r0[U::RAW], r1[U::RAW];
         S::read(img + unit_at0, 2 * part, r0);
         S::read(img + unit_at1, 2 * part + 1, r1);
-        const float before = a.residual ? *(const float*)(img + weight_pieces * 16 + ((row0 + i) & 3) * 4) : 0.f;
+        const float before = res_row ? *(const float*)(img + pieces * 16) : 0.f;
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the image is in registers: its slot is free
         if (i + 2 < R) request(i + 2);
         float v = U::dot(r0, x0, aux0) + U::dot(r1, x1, aux1);
@@ -393,6 +410,7 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
     using SL = Pairs2Slot<FMT>;
     constexpr int PD = PAIRS2_PD, NS = PD + 1, CH = SL::CH;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    QMOE_STAMP(0, 7);
     const int lane = threadIdx.x & 63, wave = uniform((int)(threadIdx.x >> 6));
     // More than four tokens are cut into groups of up to four; the workgroups are dealt out to the
     // groups in turn, and each group is a step of its own on its share of the chip: `a`, `x`, `wg` and
@@ -736,16 +754,16 @@ static bool down2_plan(const qmoe_moe_args& m, const DecodeBuffers& w, int cus, 
     a.ppr = (b.d_ff >> 8) * pp4;
     a.pps = has_shared ? (m.d_ff_shared >> 8) * pp4 : 0;
     a.ppr_magic = magic_of(a.ppr);
-    if (m.residual && ((uintptr_t)m.residual % 16 || b.d_model % 4)) return false;
-    const int pieces = m.top_k * a.ppr + a.pps + (m.residual ? 1 : 0);
+    if (m.residual && (uintptr_t)m.residual % 4) return false;
+    const int pieces = m.top_k * a.ppr + a.pps;
     a.ci = (pieces + 63) / 64;
-    a.image = pieces * 16;
+    a.image = pieces * 16 + 16;   // (+ the residual's value)
     const int floats = m.top_k * b.d_ff + (has_shared ? m.d_ff_shared : 0);
     const int chunks = (floats / 4 + 63) / 64;
     a.ch = (chunks + D2_WAVES - 1) / D2_WAVES;
     if (a.ci > DOWN2_CI || a.ch > DOWN2_CH) return false;
     a.hbytes = chunks * 1024;
-    if (a.hbytes + D2_WAVES * 768 + 1024 + D2_WAVES * 2 * a.image > D2_LDS) return false;
+    if (a.hbytes + D2_WAVES * 256 + 1024 + D2_WAVES * 2 * a.image > D2_LDS) return false;
     a.down = (const uint8_t*)b.down;
     a.down_stride = b.down_stride;
     a.shared_down = (const uint8_t*)m.shared_down_w;

@@ -100,6 +100,115 @@ __global__ __launch_bounds__(256) void norm_router_kernel(const float* __restric
     }
 }
 
+// The same for rows of up to 4096 columns, cut finer: a workgroup of eight waves owns two experts,
+// four waves each, a wave one quarter of the row.  Everything a wave needs -- its quarter of the
+// router row, of gamma and of up to four tokens -- is requested at once and kept in registers, so
+// the launch is one round trip to memory (the router row comes from HBM) plus two meetings in LDS:
+// the quarters' sums of squares, then the quarters' dot products, added in quarter order.
+static constexpr int FRONT2_THREADS = 512, FRONT2_TOKENS = 4, FRONT2_ITERS = 4;
+
+template <bool NORM>
+__global__ __launch_bounds__(FRONT2_THREADS) void norm_router_quarters_kernel(const float* __restrict__ x, int tokens, int d,
+                                                                             const float* __restrict__ gamma, float eps,
+                                                                             const float* __restrict__ w, const float* __restrict__ bias,
+                                                                             int n_experts, float* __restrict__ normalized,
+                                                                             float* __restrict__ logits) {
+    __shared__ float ss[8][FRONT2_TOKENS], dp[8][FRONT2_TOKENS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int half = wave >> 2, q = wave & 3;
+    const int e = blockIdx.x * 2 + half;
+    const bool live = e < n_experts;
+    const float* const wrow = w + (size_t)(live ? e : 0) * d;
+    const int qd = ((d / 4 + 3) / 4) * 4;                       // columns of a quarter (a multiple of four)
+    const int c_lo = q * qd, c_hi = c_lo + qd < d ? c_lo + qd : d;
+    // this block's share of the columns of `normalized`
+    const int per_block = ((d / 4 + gridDim.x - 1) / gridDim.x) * 4;
+    const int n0 = blockIdx.x * per_block, n1 = n0 + per_block < d ? n0 + per_block : d;
+    float4 r[FRONT2_ITERS], g[FRONT2_ITERS];
+#pragma unroll
+    for (int it = 0; it < FRONT2_ITERS; ++it) {
+        const int i = c_lo + 4 * lane + 256 * it;
+        const bool in = i < c_hi;
+        r[it] = in ? ldg<float4>(wrow + i) : make_float4(0, 0, 0, 0);
+        g[it] = (NORM && in) ? ldg<float4>(gamma + i) : make_float4(1, 1, 1, 1);
+    }
+    for (int t0 = 0; t0 < tokens; t0 += FRONT2_TOKENS) {
+        const int nt = tokens - t0 < FRONT2_TOKENS ? tokens - t0 : FRONT2_TOKENS;
+        float4 v[FRONT2_TOKENS][FRONT2_ITERS];
+#pragma unroll
+        for (int j = 0; j < FRONT2_TOKENS; ++j)
+#pragma unroll
+            for (int it = 0; it < FRONT2_ITERS; ++it) {
+                const int i = c_lo + 4 * lane + 256 * it;
+                v[j][it] = (i < c_hi && j < nt) ? ldg<float4>(x + (size_t)(t0 + j) * d + i) : make_float4(0, 0, 0, 0);
+            }
+        float inv[FRONT2_TOKENS];
+        if (NORM) {
+#pragma unroll
+            for (int j = 0; j < FRONT2_TOKENS; ++j) {
+                float s = 0.f;
+#pragma unroll
+                for (int it = 0; it < FRONT2_ITERS; ++it)
+                    s += (v[j][it].x * v[j][it].x + v[j][it].y * v[j][it].y) + (v[j][it].z * v[j][it].z + v[j][it].w * v[j][it].w);
+                s = wave_sum(s);
+                if (lane == 0) ss[wave][j] = s;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < FRONT2_TOKENS; ++j) {
+                const float total = ((ss[4 * half][j] + ss[4 * half + 1][j]) + ss[4 * half + 2][j]) + ss[4 * half + 3][j];
+                inv[j] = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(total, (float)d) + eps));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FRONT2_TOKENS; ++j) {
+            float acc = 0.f;
+#pragma unroll
+            for (int it = 0; it < FRONT2_ITERS; ++it) {
+                const float4 a = v[j][it];
+                if (NORM)
+                    acc += (mul_unfused(mul_unfused(a.x, inv[j]), g[it].x) * r[it].x + mul_unfused(mul_unfused(a.y, inv[j]), g[it].y) * r[it].y) +
+                           (mul_unfused(mul_unfused(a.z, inv[j]), g[it].z) * r[it].z + mul_unfused(mul_unfused(a.w, inv[j]), g[it].w) * r[it].w);
+                else
+                    acc += (a.x * r[it].x + a.y * r[it].y) + (a.z * r[it].z + a.w * r[it].w);
+            }
+            acc = wave_sum(acc);
+            if (lane == 0) dp[wave][j] = acc;
+        }
+        __syncthreads();
+        if (q == 0 && lane < nt && live) {
+            const float sum = ((dp[4 * half][lane] + dp[4 * half + 1][lane]) + dp[4 * half + 2][lane]) + dp[4 * half + 3][lane];
+            logits[(size_t)(t0 + lane) * n_experts + e] = sum + (bias ? bias[e] : 0.0f);
+        }
+        if (NORM) {
+            // (the inverse RMS of a token is the same in every wave: any wave's copy will do)
+            for (int idx = threadIdx.x; idx < nt * (per_block / 4); idx += FRONT2_THREADS) {
+                const int j = idx / (per_block / 4), i = n0 + 4 * (idx % (per_block / 4));
+                if (i < n1) {
+                    const float4 xv = ldg<float4>(x + (size_t)(t0 + j) * d + i), gv = ldg<float4>(gamma + i);
+                    const float total = ((ss[0][j] + ss[1][j]) + ss[2][j]) + ss[3][j];
+                    const float iv = __fdiv_rn(1.0f, __fsqrt_rn(__fdiv_rn(total, (float)d) + eps));
+                    stg<float4>(normalized + (size_t)(t0 + j) * d + i,
+                                make_float4(mul_unfused(mul_unfused(xv.x, iv), gv.x), mul_unfused(mul_unfused(xv.y, iv), gv.y),
+                                            mul_unfused(mul_unfused(xv.z, iv), gv.z), mul_unfused(mul_unfused(xv.w, iv), gv.w)));
+                }
+            }
+        }
+        __syncthreads();   // the LDS cells are written again by the next group of tokens
+    }
+}
+
+template <bool NORM>
+static void launch_norm_router(const float* x, int tokens, int d, const float* gamma, float eps, const float* w, const float* bias,
+                               int n_experts, float* normalized, float* logits, hipStream_t s) {
+    if (d <= 4 * 256 * FRONT2_ITERS)
+        hipLaunchKernelGGL(norm_router_quarters_kernel<NORM>, dim3((n_experts + 1) / 2), dim3(FRONT2_THREADS), 0, s, x, tokens, d, gamma,
+                           eps, w, bias, n_experts, normalized, logits);
+    else
+        hipLaunchKernelGGL(norm_router_kernel<NORM>, dim3((n_experts + 3) / 4), dim3(256), 0, s, x, tokens, d, gamma, eps, w, bias,
+                           n_experts, normalized, logits);
+}
+
 }  // namespace qmoe
 
 using namespace qmoe;
@@ -114,8 +223,7 @@ extern "C" int qmoe_norm_router(const float* x, int tokens, int d_model, const f
     if (d_model % 4) return fail(QMOE_EUNSUPPORTED, "qmoe_norm_router: d_model=%d is not a multiple of 4", d_model);
     if (((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)router_w | (uintptr_t)normalized) % 16)
         return fail(QMOE_EUNSUPPORTED, "qmoe_norm_router: x, gamma, router_w and normalized must be 16-byte aligned");
-    hipLaunchKernelGGL(norm_router_kernel<true>, dim3((n_experts + 3) / 4), dim3(256), 0, (hipStream_t)stream, x, tokens, d_model,
-                       gamma, eps, router_w, router_b, n_experts, normalized, logits);
+    launch_norm_router<true>(x, tokens, d_model, gamma, eps, router_w, router_b, n_experts, normalized, logits, (hipStream_t)stream);
     return check_launch("qmoe_norm_router");
 }
 
@@ -127,7 +235,7 @@ extern "C" int qmoe_router_logits(const float* x, int tokens, int d_model, const
     if (d_model % 4) return fail(QMOE_EUNSUPPORTED, "qmoe_router_logits: d_model=%d is not a multiple of 4", d_model);
     if (((uintptr_t)x | (uintptr_t)router_w) % 16)
         return fail(QMOE_EUNSUPPORTED, "qmoe_router_logits: x and router_w must be 16-byte aligned");
-    hipLaunchKernelGGL(norm_router_kernel<false>, dim3((n_experts + 3) / 4), dim3(256), 0, (hipStream_t)stream, x, tokens,
-                       d_model, (const float*)nullptr, 0.0f, router_w, router_b, n_experts, (float*)nullptr, logits);
+    launch_norm_router<false>(x, tokens, d_model, (const float*)nullptr, 0.0f, router_w, router_b, n_experts, (float*)nullptr, logits,
+                              (hipStream_t)stream);
     return check_launch("qmoe_router_logits");
 }
