@@ -358,6 +358,51 @@ def moe_decode_extra(torch, lib, device, fmt, tokens, steps, warmup, layer_half=
             "tokens_per_s": round(tokens / per_step, 1), "host_ms_per_step": round(wall / steps * 1e3, 4)}
 
 
+def grouped_decode_extra(torch, lib, device, fmt, count, steps, warmup):
+    """The reference's decode entry point (grouped_quantized_experts_forward): one token through
+    `count` expert handles of the 512-expert layer's shape (2048 -> 512 -> 2048), no router and no
+    shared expert; handles given as a host list per step (qmoe_grouped_decode_listed).  Cold: steps
+    rotate over four banks and 48 different selections, as the MoE decode steps do."""
+    e, d, f = 512, 2048, 512
+    gen = torch.Generator(device=device)
+    gen.manual_seed(11)
+    banks = [tuple(device_blocks(torch, fmt, e * n, kk, gen, device) for n, kk in ((f, d), (f, d), (d, f))) for _ in range(4)]
+    row = {"g": weight_bytes(fmt, f, d), "d": weight_bytes(fmt, d, f)}
+    x = torch.randn((1, d), device=device, generator=gen)
+    routes = torch.rand(count, device=device, generator=gen)
+    out = torch.empty((1, d), device=device)
+    workspace = torch.empty(count * (f + d + 8), device=device)
+    import numpy as np
+    cycle = 4 * 48
+    rng = np.random.default_rng(5)
+    tables = []
+    for i in range(cycle):
+        g, u, dn = banks[i % 4]
+        chosen = np.sort(rng.choice(e, count, replace=False))
+        ptrs = []
+        for j in chosen:
+            ptrs += [g.data_ptr() + int(j) * row["g"], u.data_ptr() + int(j) * row["g"], dn.data_ptr() + int(j) * row["d"]]
+        tables.append((ctypes.c_void_p * (3 * count))(*ptrs))
+    from mylocal_llm_amd import _lib
+    state = {"i": 0}
+    fid = _lib.FORMAT_ID[fmt]
+
+    def fn(stream):
+        table = tables[state["i"] % cycle]
+        state["i"] += 1
+        rc = lib.qmoe_grouped_decode_listed(x.data_ptr(), ctypes.cast(table, ctypes.c_void_p), count, fid, fid, fid, d, f,
+                                            routes.data_ptr(), 1, None, out.data_ptr(), workspace.data_ptr(), stream)
+        if rc:
+            raise RuntimeError(lib.qmoe_last_error().decode())
+
+    wall, ms = time_steps(torch, fn, steps, warmup)
+    nbytes = count * 3 * row["g"]
+    per_step = ms / steps * 1e-3
+    return {"workload": f"grouped_decode_{fmt}_E{count}", "residency": "cold: 4 banks x 48 selections in rotation",
+            "ms_per_step": round(ms / steps, 4), "weight_bytes": int(nbytes), "GBps": round(nbytes / per_step / 1e9, 1),
+            "frac_hbm_peak": round(nbytes / per_step / 1e9 / HBM_PEAK_GBS, 4), "host_ms_per_step": round(wall / steps * 1e3, 4)}
+
+
 def moe_prefill_extra(torch, lib, device, fmt, tokens, steps, warmup):
     """512-expert top-10 MoE step at prefill size: Zipf(1.1) expert popularity over a seeded
     permutation, routing from logits, token-tile MFMA GEMMs, fp32 output [T, 2048]."""
@@ -469,7 +514,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_timeline", "moe_layer_half", "layer_few_tokens", "read_probe",
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_timeline", "moe_layer_half", "grouped_decode", "layer_few_tokens", "read_probe",
                                        "layer_q6_k", "layer_q5_k", "layer_q4_k", "layer_by_dependency"], default=None,
                     help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -497,6 +542,9 @@ def main():
         return
     if args.only == "moe_timeline":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, timeline=True) for t in (1, 4)], indent=1))
+        return
+    if args.only == "grouped_decode":
+        print(json.dumps([grouped_decode_extra(torch, lib, device, fmt, 10, max(8, args.steps), args.warmup) for fmt in ("Q8_0", "Q6_K")]))
         return
     if args.only == "moe_decode_hot":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, hot=True) for t in (1, 4, 16)]))
@@ -570,6 +618,8 @@ def main():
         for fmt, tokens in (("Q8_0", 1), ("Q8_0", 4), ("Q8_0", 16), ("Q6_K", 1)):
             extras.append(moe_decode_extra(torch, lib, device, fmt, tokens, max(8, args.steps), 3))
             torch.cuda.empty_cache()
+        extras.append(grouped_decode_extra(torch, lib, device, "Q8_0", 10, max(8, args.steps), 3))
+        torch.cuda.empty_cache()
         extras.append(moe_decode_extra(torch, lib, device, "Q8_0", 1, max(8, args.steps), 3, hot=True))
         torch.cuda.empty_cache()
         for tokens in (1, 4):

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define QMOE_ABI_VERSION 4
+#define QMOE_ABI_VERSION 5
 
 /* Packed formats.  Ids 0..5 are the reference's (_FORMAT_ID,
  * mini_llm/ops/quantized_linear.py:34 and native_packed_cpu.cpp:12).  BF16 has no
@@ -163,6 +163,22 @@ int qmoe_grouped_decode(const float* x, const void* const* table, int n_rows,
                         int gate_fmt, int up_fmt, int down_fmt, int d_model, int d_ff,
                         const float* routes, int64_t route_stride, const int32_t* slots,
                         float* out, float* workspace, void* stream);
+
+/* qmoe_grouped_decode for a caller that holds the expert table on the HOST (as the reference's
+ * wrapper does before it uploads it, mini_llm/ops/grouped_quantized_experts.py:180-186): `experts`
+ * is a HOST array of n_rows x 3 device pointers (gate, up, down), `slots` a HOST array of n_rows
+ * route positions or NULL; both are read before the call returns and travel in the kernel
+ * arguments, so the call makes no host-to-device copy.  Up to 16 experts (more: QMOE_EUNSUPPORTED,
+ * use the device-table form).  Same result as qmoe_grouped_decode: the same ordered sum of stored
+ * products.  Shapes the streamed decode kernels take (all formats Q8_0 / Q4_K / Q5_K / Q6_K with
+ * gate_fmt == up_fmt, d_model a multiple of 256 up to 2048, d_ff a power-of-two multiple of 256,
+ * n_rows * d_ff / 128 <= 48) run on them in two launches; any other shape runs the general kernels.
+ * workspace: fp32 n_rows * (d_ff + d_model + 8) elements, 16-byte aligned.  No counterpart in the
+ * reference beyond the call it replaces. */
+int qmoe_grouped_decode_listed(const float* x, const void* const* experts, int n_rows,
+                               int gate_fmt, int up_fmt, int down_fmt, int d_model, int d_ff,
+                               const float* routes, int64_t route_stride, const int32_t* slots,
+                               float* out, float* workspace, void* stream);
 
 /* Arguments of one MoE step over T tokens.  Host struct. */
 typedef struct qmoe_moe_args {

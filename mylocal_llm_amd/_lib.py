@@ -43,7 +43,7 @@ class MoeArgs(ctypes.Structure):
                 ("out", _P), ("out_dtype", _I), ("out_weights", _P), ("out_ids", _P), ("residual", _P), ("status_out", _P)]
 
 
-ABI_VERSION = 4   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
+ABI_VERSION = 5   # QMOE_ABI_VERSION of include/qmoe.h this binding was written against
 
 _SIGNATURES = {
     "qmoe_abi_version": ([], _I),
@@ -59,6 +59,7 @@ _SIGNATURES = {
     "qmoe_expert": ([_P, _I, _P, _I, _P, _I, _I, _I, _P, _I, _I, _P, _I, _P, _P], _I),
     "qmoe_router_topk": ([_P, _I, _I, _I, _F, _I, _P, _P, _P], _I),
     "qmoe_grouped_decode": ([_P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _P, _P], _I),
+    "qmoe_grouped_decode_listed": ([_P, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _P, _P, _P, _P], _I),
     "qmoe_moe_workspace_bytes": ([_I, _I, _I, _I, _I, _I], _SZ),
     "qmoe_moe_forward": ([ctypes.POINTER(MoeArgs), _P, _SZ, _P], _I),
     "qmoe_norm_router": ([_P, _I, _I, _P, _F, _P, _P, _I, _P, _P, _P], _I),

@@ -123,11 +123,29 @@ __device__ __forceinline__ void route_token(const DecodeRouteArgs& a, int t, boo
     }
 }
 
+// The experts of a single token given one by one instead of as ids into a bank (the grouped
+// decode call): pointers and route positions travel in the kernel arguments, in the order the
+// experts are summed.  count == 0: no table, the step addresses a bank.
+static constexpr int LISTED_MAX = 16;
+struct ListedExperts {
+    const uint8_t* gate[LISTED_MAX];
+    const uint8_t* up[LISTED_MAX];
+    const uint8_t* down[LISTED_MAX];
+    int slot[LISTED_MAX];     // position of each expert's weight in `routes`
+    const float* routes;      // device, fp32
+    int64_t route_stride;     // elements between route positions
+    int count;
+};
+
 // The LDS-DMA kernels of the decode step (qmoe_decode2.hip): routing + gate/up for up to four
 // tokens, down + combine for up to sixteen; each says whether it takes a step's shapes.
 bool decode2_pairs_supported(const qmoe_moe_args& m);
-int decode2_pairs_launch(const qmoe_moe_args& m, const DecodeRouteArgs& r, hipStream_t s);
+int decode2_pairs_launch(const qmoe_moe_args& m, const DecodeRouteArgs& r, hipStream_t s, const ListedExperts* listed = nullptr);
 bool decode2_down_supported(const qmoe_moe_args& m, const DecodeBuffers& w);
-int decode2_down_launch(const qmoe_moe_args& m, const DecodeBuffers& w, hipStream_t s);
+int decode2_down_launch(const qmoe_moe_args& m, const DecodeBuffers& w, hipStream_t s, const ListedExperts* listed = nullptr);
+// A single token through listed experts: out[d] = sum in list order of fp32(down_e(swiglu_e(x))[d] * route_e);
+// QMOE_EUNSUPPORTED (nothing launched) for shapes the two kernels do not take.
+int decode2_listed(const float* x, const ListedExperts& listed, int gate_fmt, int up_fmt, int down_fmt, int d_model, int d_ff,
+                   float* out, float* workspace, hipStream_t s);
 
 }  // namespace qmoe

@@ -150,7 +150,7 @@ struct Down2Args {
 // while one is multiplied.
 // LDS: [staged activations | per wave: expert ids | dump | per wave: two row images]
 template <int FMT>
-__global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a) {
+__global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a, const ListedExperts listed) {
     using U = Unit64<FMT>;
     using S = SpanFmt<FMT>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -231,7 +231,8 @@ __global__ __launch_bounds__(D2_THREADS, 1) void down2_kernel(const Down2Args a)
     for (int c = 0; c < DOWN2_CI; ++c)
         if ((is_routed >> c) & 1u) {
             const int e = tab_ids[(slot_of >> (4 * c)) & 15u];
-            src[c] += (int64_t)(e >= 0 ? e : 0) * a.down_stride;
+            if (listed.count) src[c] = listed.down[e >= 0 && e < listed.count ? e : 0] + (src[c] - a.down);   // ("ids" are list positions)
+            else src[c] += (int64_t)(e >= 0 ? e : 0) * a.down_stride;
         }
     // With a residual, its value of the row travels with the row, behind the image (an ordinary
     // load here would make the compiler wait for everything in flight).
@@ -404,7 +405,7 @@ template <int FMT> struct Pairs2Slot {
 
 // LDS: [activations fp32, swizzled | sorted ids per token | dump | rings: 8 waves x 3 slots]
 template <int FMT>
-__global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRouteArgs step, const Pairs2Shape shape) {
+__global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRouteArgs step, const Pairs2Shape shape, const ListedExperts listed) {
     using U = Unit64<FMT>;
     using S = SpanFmt<FMT>;
     using SL = Pairs2Slot<FMT>;
@@ -485,7 +486,12 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
             it.r0 = (int)(q - tj * (uint32_t)x.ipe) * x.ri;
             it.t = (int)t;
             const int64_t e = uniform64(sid[t * 32 + (tj - t * (uint32_t)k)]);
-            if (e >= 0) {
+            if (e >= 0 && listed.count) {   // (listed experts: the "id" is the list position)
+                it.g = listed.gate[e] + (int64_t)it.r0 * rb;
+                it.u = listed.up[e] + (int64_t)it.r0 * rb;
+                it.y = a.h + (size_t)tj * a.f + it.r0;
+                it.live = true;
+            } else if (e >= 0) {
                 it.g = a.gate + e * a.gate_stride + (int64_t)it.r0 * rb;
                 it.u = a.up + e * a.up_stride + (int64_t)it.r0 * rb;
                 it.y = a.h + (size_t)tj * a.f + it.r0;
@@ -549,8 +555,13 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
     int64_t id = 0;
     if (selects && !from_logits) {
         const int kk = lane < k ? lane : k - 1;
-        id = a.in_ids[(size_t)token * k + kk];
-        weight = a.in_weights[(size_t)token * k + kk];
+        if (listed.count) {   // listed experts: position kk of the list, its weight from the caller's routes
+            id = kk;
+            weight = listed.routes[(int64_t)listed.slot[kk] * listed.route_stride];
+        } else {
+            id = a.in_ids[(size_t)token * k + kk];
+            weight = a.in_weights[(size_t)token * k + kk];
+        }
         asm volatile("" ::"v"((uint32_t)id), "v"((uint32_t)((uint64_t)id >> 32)), "v"(weight) : "memory");
     }
     // ... or the router row, into the second slot of this wave's ring (and on into the third)
@@ -655,7 +666,7 @@ __global__ __launch_bounds__(D2_THREADS, 1) void pairs2_kernel(const DecodeRoute
         // bank, or an expert the token has named in an earlier slot already, contributes nothing.
         int rank = 0;
         bool again = false;
-        for (int j = 0; j < k; ++j) {
+        for (int j = 0; j < k; ++j) {   // (listed experts: ids are 0 .. k - 1, rank = position, nothing repeats)
             const int64_t other = readlane_i64(id, j);
             rank += (other < id) || (other == id && j < lane);
             again |= other == id && j < lane;
@@ -785,7 +796,7 @@ static bool down2_plan(const qmoe_moe_args& m, const DecodeBuffers& w, int cus, 
 }
 
 template <int FMT>
-static int down2_launch_as(const Down2Args& a, int tokens, hipStream_t s) {
+static int down2_launch_as(const Down2Args& a, int tokens, const ListedExperts& listed, hipStream_t s) {
     static bool configured = false;   // (benign if two threads both set it)
     if (!configured) {
         if (hipFuncSetAttribute((const void*)down2_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, D2_LDS) != hipSuccess)
@@ -793,20 +804,22 @@ static int down2_launch_as(const Down2Args& a, int tokens, hipStream_t s) {
         configured = true;
     }
     const int per_wg = D2_WAVES * a.rows;
-    hipLaunchKernelGGL(down2_kernel<FMT>, dim3((a.d + per_wg - 1) / per_wg, tokens), dim3(D2_THREADS), D2_LDS, s, a);
+    hipLaunchKernelGGL(down2_kernel<FMT>, dim3((a.d + per_wg - 1) / per_wg, tokens), dim3(D2_THREADS), D2_LDS, s, a, listed);
     return check_launch("qmoe_moe_forward(down)");
 }
 
 bool decode2_down_supported(const qmoe_moe_args& m, const DecodeBuffers& w) { return down2_plan(m, w, stream_grid() / 2, nullptr); }
 
-int decode2_down_launch(const qmoe_moe_args& m, const DecodeBuffers& w, hipStream_t s) {
+int decode2_down_launch(const qmoe_moe_args& m, const DecodeBuffers& w, hipStream_t s, const ListedExperts* listed) {
+    ListedExperts l{};
+    if (listed) l = *listed;
     Down2Args a;
     if (!down2_plan(m, w, stream_grid() / 2, &a)) return fail(QMOE_EUNSUPPORTED, "MoE decode (down): shape not taken");
     switch (m.bank.down_fmt) {
-    case QMOE_FMT_Q8_0: return down2_launch_as<QMOE_FMT_Q8_0>(a, m.tokens, s);
-    case QMOE_FMT_Q6_K: return down2_launch_as<QMOE_FMT_Q6_K>(a, m.tokens, s);
-    case QMOE_FMT_Q5_K: return down2_launch_as<QMOE_FMT_Q5_K>(a, m.tokens, s);
-    default: return down2_launch_as<QMOE_FMT_Q4_K>(a, m.tokens, s);
+    case QMOE_FMT_Q8_0: return down2_launch_as<QMOE_FMT_Q8_0>(a, m.tokens, l, s);
+    case QMOE_FMT_Q6_K: return down2_launch_as<QMOE_FMT_Q6_K>(a, m.tokens, l, s);
+    case QMOE_FMT_Q5_K: return down2_launch_as<QMOE_FMT_Q5_K>(a, m.tokens, l, s);
+    default: return down2_launch_as<QMOE_FMT_Q4_K>(a, m.tokens, l, s);
     }
 }
 
@@ -851,7 +864,7 @@ static bool pairs2_plan(const qmoe_moe_args& m, int waves, Pairs2Shape* out) {
 }
 
 template <int FMT>
-static int pairs2_launch_as(const DecodeRouteArgs& r, const Pairs2Shape& x, int grid, hipStream_t s) {
+static int pairs2_launch_as(const DecodeRouteArgs& r, const Pairs2Shape& x, int grid, const ListedExperts& listed, hipStream_t s) {
     static bool configured = false;   // (benign if two threads both set it)
     if (!configured) {
         if (hipFuncSetAttribute((const void*)pairs2_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, D2_LDS) != hipSuccess)
@@ -860,22 +873,80 @@ static int pairs2_launch_as(const DecodeRouteArgs& r, const Pairs2Shape& x, int 
     }
     static_assert(PAIRS2_MAX_TOKENS * 2048 * 4 + PAIRS2_MAX_TOKENS * 32 * 8 + PAIRS2_MAX_TOKENS * sizeof(RouteShare) + 1024 +
                   D2_WAVES * (PAIRS2_PD + 1) * Pairs2Slot<FMT>::BYTES <= D2_LDS, "LDS layout of the gate/up kernel");
-    hipLaunchKernelGGL(pairs2_kernel<FMT>, dim3(grid), dim3(D2_THREADS), D2_LDS, s, r, x);
+    hipLaunchKernelGGL(pairs2_kernel<FMT>, dim3(grid), dim3(D2_THREADS), D2_LDS, s, r, x, listed);
     return check_launch("qmoe_moe_forward(route + gate/up)");
 }
 
 bool decode2_pairs_supported(const qmoe_moe_args& m) { return pairs2_plan(m, (stream_grid() / 2) * D2_WAVES, nullptr); }
 
-int decode2_pairs_launch(const qmoe_moe_args& m, const DecodeRouteArgs& r, hipStream_t s) {
+int decode2_pairs_launch(const qmoe_moe_args& m, const DecodeRouteArgs& r, hipStream_t s, const ListedExperts* listed) {
+    ListedExperts l{};
+    if (listed) l = *listed;
     const int grid = stream_grid() / 2;
     Pairs2Shape x;
     if (!pairs2_plan(m, grid * D2_WAVES, &x)) return fail(QMOE_EUNSUPPORTED, "MoE decode (gate/up): shape not taken");
     switch (m.bank.gate_fmt) {
-    case QMOE_FMT_Q8_0: return pairs2_launch_as<QMOE_FMT_Q8_0>(r, x, grid, s);
-    case QMOE_FMT_Q6_K: return pairs2_launch_as<QMOE_FMT_Q6_K>(r, x, grid, s);
-    case QMOE_FMT_Q5_K: return pairs2_launch_as<QMOE_FMT_Q5_K>(r, x, grid, s);
-    default: return pairs2_launch_as<QMOE_FMT_Q4_K>(r, x, grid, s);
+    case QMOE_FMT_Q8_0: return pairs2_launch_as<QMOE_FMT_Q8_0>(r, x, grid, l, s);
+    case QMOE_FMT_Q6_K: return pairs2_launch_as<QMOE_FMT_Q6_K>(r, x, grid, l, s);
+    case QMOE_FMT_Q5_K: return pairs2_launch_as<QMOE_FMT_Q5_K>(r, x, grid, l, s);
+    default: return pairs2_launch_as<QMOE_FMT_Q4_K>(r, x, grid, l, s);
     }
+}
+
+
+int decode2_listed(const float* x, const ListedExperts& listed, int gate_fmt, int up_fmt, int down_fmt, int d_model, int d_ff,
+                   float* out, float* workspace, hipStream_t s) {
+    const int e = listed.count;
+    if (e < 1 || e > LISTED_MAX) return fail(QMOE_EUNSUPPORTED, "listed experts: %d experts (1..%d)", e, LISTED_MAX);
+    // the step as the two kernels see it: one token, top_k = the list, "expert ids" = list positions
+    qmoe_moe_args m{};
+    m.hidden = x;
+    m.hidden_dtype = QMOE_DT_F32;
+    m.tokens = 1;
+    m.top_k = e;
+    m.bank.gate = listed.gate[0];
+    m.bank.up = listed.up[0];
+    m.bank.down = listed.down[0];
+    m.bank.gate_fmt = gate_fmt;
+    m.bank.up_fmt = up_fmt;
+    m.bank.down_fmt = down_fmt;
+    m.bank.n_experts = e;
+    m.bank.d_model = d_model;
+    m.bank.d_ff = d_ff;
+    m.out = out;
+    m.out_dtype = QMOE_DT_F32;
+    const int align_gu = gate_fmt == QMOE_FMT_Q6_K ? 2 : 16, align_d = down_fmt == QMOE_FMT_Q6_K ? 2 : 16;
+    for (int i = 0; i < e; ++i)
+        if ((uintptr_t)listed.gate[i] % align_gu || (uintptr_t)listed.up[i] % align_gu || (uintptr_t)listed.down[i] % align_d)
+            return fail(QMOE_EUNSUPPORTED, "listed experts: expert %d is not aligned for the streaming kernels", i);
+    // workspace: [e * d_ff] SwiGLU activations, then the routing as the down kernel reads it
+    DecodeBuffers w{};
+    w.h = workspace;
+    w.hs = workspace;   // (no shared expert: never read)
+    float* const tail = workspace + (size_t)e * d_ff;
+    w.sorted_ids = (int*)tail;
+    w.sorted_w = tail + LISTED_MAX;
+    w.sig = tail + 2 * LISTED_MAX;
+    if ((size_t)e * d_model < 3 * LISTED_MAX) return fail(QMOE_EUNSUPPORTED, "listed experts: workspace too small for the routing");
+    if (!decode2_pairs_supported(m) || !decode2_down_supported(m, w)) return fail(QMOE_EUNSUPPORTED, "listed experts: shape not taken");
+    DecodeRouteArgs r{};
+    r.sorted_ids = w.sorted_ids;
+    r.sorted_w = w.sorted_w;
+    r.sig = w.sig;
+    r.hidden = x;
+    r.gate = listed.gate[0];
+    r.up = listed.up[0];
+    r.h = w.h;
+    r.hs = w.hs;
+    r.n_experts = e;
+    r.k = e;
+    r.d = d_model;
+    r.f = d_ff;
+    r.fmt = gate_fmt;
+    r.xdt = QMOE_DT_F32;
+    r.tokens = 1;
+    if (int rc = decode2_pairs_launch(m, r, s, &listed)) return rc;
+    return decode2_down_launch(m, w, s, &listed);
 }
 
 }  // namespace qmoe

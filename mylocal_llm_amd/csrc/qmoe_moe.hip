@@ -9,6 +9,7 @@
 //   pos_of[T*k]       sorted position of assignment (t, slot)
 //   hidden_act[A, F]  fp32 SwiGLU activations, terms[A, D] fp32 weighted expert outputs
 // with A = T*k.  Nothing is read back by the host.
+#include "qmoe_decode.hpp"
 #include "qmoe_gemm.hpp"
 #include "qmoe_rowdot.hpp"
 #include <mutex>
@@ -760,6 +761,65 @@ int qmoe_grouped_decode(const float* x, const void* const* table, int n_rows, in
 }
 
 }  // extern "C"
+
+namespace qmoe {
+// The listed experts' pointers and route positions from the kernel arguments into device memory
+// (for the general kernels, which read a device table): no host-to-device copy is involved.
+__global__ void listed_upload_kernel(const ListedExperts l, const void** table, int32_t* slots) {
+    const int i = threadIdx.x;
+    if (i < l.count) {
+        table[3 * i] = l.gate[i];
+        table[3 * i + 1] = l.up[i];
+        table[3 * i + 2] = l.down[i];
+        slots[i] = l.slot[i];
+    }
+}
+}  // namespace qmoe
+
+extern "C" int qmoe_grouped_decode_listed(const float* x, const void* const* experts, int n_rows, int gate_fmt, int up_fmt,
+                                          int down_fmt, int d_model, int d_ff, const float* routes, int64_t route_stride,
+                                          const int32_t* slots, float* out, float* workspace, void* stream) {
+    const char* who = "qmoe_grouped_decode_listed";
+    if (!x || !experts || !routes || !out) return fail(QMOE_EINVAL, "%s: null pointer", who);
+    if (!workspace || (uintptr_t)workspace % 16) return fail(QMOE_EWORKSPACE, "%s: workspace of E*(d_ff+d_model+8) floats (16-byte aligned) required", who);
+    if (n_rows < 1) return fail(QMOE_EINVAL, "%s: expert rows %d", who, n_rows);
+    if (n_rows > LISTED_MAX) return fail(QMOE_EUNSUPPORTED, "%s: %d experts exceed the %d a host list carries; use qmoe_grouped_decode", who, n_rows, LISTED_MAX);
+    if (d_model < 1 || d_ff < 1) return fail(QMOE_EINVAL, "%s: dimensions must be positive", who);
+    const int fmts[3] = {gate_fmt, up_fmt, down_fmt};
+    const int ks[3] = {d_model, d_model, d_ff};
+    for (int i = 0; i < 3; ++i) {
+        if (!block_elems(fmts[i])) return fail(QMOE_EINVAL, "%s: unknown packed format id %d", who, fmts[i]);
+        if (!format_implemented(fmts[i])) return fail(QMOE_EUNSUPPORTED, "%s: packed format id %d has no kernel", who, fmts[i]);
+        if (ks[i] % block_elems(fmts[i])) return fail(QMOE_EINVAL, "%s: projection K=%d is not a block multiple", who, ks[i]);
+    }
+    ListedExperts l{};
+    for (int i = 0; i < n_rows; ++i) {
+        l.gate[i] = (const uint8_t*)experts[3 * i];
+        l.up[i] = (const uint8_t*)experts[3 * i + 1];
+        l.down[i] = (const uint8_t*)experts[3 * i + 2];
+        if (!l.gate[i] || !l.up[i] || !l.down[i]) return fail(QMOE_EINVAL, "%s: expert %d has a null projection", who, i);
+        if ((uintptr_t)l.gate[i] % 2 || (uintptr_t)l.up[i] % 2 || (uintptr_t)l.down[i] % 2)
+            return fail(QMOE_EINVAL, "%s: packed weights must be 2-byte aligned", who);
+        l.slot[i] = slots ? slots[i] : i;
+        if (l.slot[i] < 0) return fail(QMOE_EINVAL, "%s: negative route position", who);
+    }
+    l.routes = routes;
+    l.route_stride = route_stride;
+    l.count = n_rows;
+    hipStream_t s = (hipStream_t)stream;
+    if ((uintptr_t)x % 16 == 0) {
+        const int rc = decode2_listed(x, l, gate_fmt, up_fmt, down_fmt, d_model, d_ff, out, workspace, s);
+        if (rc != QMOE_EUNSUPPORTED) return rc;
+    }
+    // any other shape: the table goes to the end of the workspace, then the general kernels
+    float* const tail = workspace + (size_t)n_rows * ((size_t)d_ff + d_model);
+    const void** const table = (const void**)tail;
+    int32_t* const dslots = (int32_t*)(tail + 6 * (size_t)n_rows);
+    hipLaunchKernelGGL(listed_upload_kernel, dim3(1), dim3(64), 0, s, l, table, dslots);
+    if (int rc = check_launch("qmoe_grouped_decode_listed(table)")) return rc;
+    return qmoe_grouped_decode(x, (const void* const*)table, n_rows, gate_fmt, up_fmt, down_fmt, d_model, d_ff, routes, route_stride,
+                               dslots, out, workspace, stream);
+}
 
 extern "C" int qmoe_routing_plan(const int64_t* ids, const float* weights, int tokens, int top_k, int n_experts,
                                  int* offsets, int* active, int* n_active, int* order, int* sorted_token,

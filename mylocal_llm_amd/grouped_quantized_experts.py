@@ -91,27 +91,59 @@ def supports_grouped_quantized_experts(x, experts, routing_weights, *, block_k=5
     return _unsupported_reason(x, experts, routing_weights, block_k, routing_slots) is None
 
 
+# Host lists of up to this many experts travel in the kernel arguments (qmoe_grouped_decode_listed).
+_LISTED_MAX = 16
+# One scratch tensor per (device, stream) grown on demand: a decode loop calls with the same sizes
+# every token, so a call allocates nothing but its fresh output.  Work on one stream is ordered, so
+# consecutive calls may share the scratch; calls on different streams get different tensors.
+_SCRATCH = {}
+
+
+def _scratch(device, floats):
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    held = _SCRATCH.get(key)
+    if held is None or held.numel() < floats:
+        held = torch.empty(floats, dtype=torch.float32, device=device)
+        _SCRATCH[key] = held
+    return held
+
+
 def grouped_quantized_experts_forward(x, experts, routing_weights, *, block_k=512,
                                       routing_slots=None):
-    """Return a fresh FP32 [1, D] weighted expert sum on torch's current stream."""
+    """Return a fresh FP32 [1, D] weighted expert sum on torch's current stream.
+
+    Up to 16 handles (a decode step's top-k) are handed over as a host list: pointers and route
+    positions go into the kernel arguments and the scratch is reused across calls, so the call
+    uploads nothing and allocates only its output.  Longer lists build a device pointer table as the
+    reference does (mini_llm/ops/grouped_quantized_experts.py:180-186)."""
     reason = _unsupported_reason(x, experts, routing_weights, block_k, routing_slots)
     if reason is not None:
         raise ValueError(f"Unsupported grouped quantized experts: {reason}")
     e, d, f = len(experts), x.shape[1], experts[0].gate.shape[0]
-    host = np.asarray([[w.data.data_ptr() for w in (h.gate, h.up, h.down)] for h in experts], dtype=np.uint64)
-    table = torch.from_numpy(host.view(np.int64)).to(x.device, non_blocking=False)
-    slots = None
-    if routing_slots is not None:
-        slots = torch.tensor([int(s) for s in routing_slots], dtype=torch.int32).to(x.device)
-    workspace = torch.empty(e * (f + d), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    first = experts[0]
+    formats = tuple(_FORMAT_ID[w.quant_type] for w in (first.gate, first.up, first.down))
     out = torch.empty((1, d), dtype=torch.float32, device=x.device)
-    gate, up, down = experts[0].gate, experts[0].up, experts[0].down
     stride = routing_weights.stride(0)
+    pointers = [w.data.data_ptr() for h in experts for w in (h.gate, h.up, h.down)]
     with torch.cuda.device(x.device):
-        rc = _lib.load().qmoe_grouped_decode(
-            _ptr(x), _ptr(table), e, _FORMAT_ID[gate.quant_type], _FORMAT_ID[up.quant_type],
-            _FORMAT_ID[down.quant_type], d, f, _ptr(routing_weights), stride,
-            _ptr(slots) if slots is not None else ctypes.c_void_p(0),
-            _ptr(out), _ptr(workspace), _stream())
+        if e <= _LISTED_MAX:
+            table = (ctypes.c_void_p * (3 * e))(*pointers)
+            slots = (ctypes.c_int32 * e)(*(int(s) for s in routing_slots)) if routing_slots is not None else None
+            workspace = _scratch(x.device, e * (f + d + 8))
+            rc = lib.qmoe_grouped_decode_listed(
+                _ptr(x), ctypes.cast(table, ctypes.c_void_p), e, *formats, d, f, _ptr(routing_weights), stride,
+                ctypes.cast(slots, ctypes.c_void_p) if slots is not None else ctypes.c_void_p(0),
+                _ptr(out), _ptr(workspace), _stream())
+        else:
+            table = torch.from_numpy(np.asarray(pointers, dtype=np.uint64).view(np.int64)).to(x.device, non_blocking=False)
+            slots = None
+            if routing_slots is not None:
+                slots = torch.tensor([int(s) for s in routing_slots], dtype=torch.int32).to(x.device)
+            workspace = torch.empty(e * (f + d), dtype=torch.float32, device=x.device)
+            rc = lib.qmoe_grouped_decode(
+                _ptr(x), _ptr(table), e, *formats, d, f, _ptr(routing_weights), stride,
+                _ptr(slots) if slots is not None else ctypes.c_void_p(0),
+                _ptr(out), _ptr(workspace), _stream())
     _lib.check(rc, "Grouped packed experts")
     return out

@@ -209,6 +209,32 @@ def test_grouped_decode_matches_oracle(cuda, formats):
     assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("fmt", ["Q8_0", "Q6_K", "Q5_K", "Q4_K"])
+@pytest.mark.parametrize("count", [1, 10, 12, 20])
+def test_grouped_decode_at_the_decode_shape(cuda, fmt, count):
+    """A decode step's selection at the benchmark's expert shape (2048 -> 512 -> 2048): up to 16
+    handles travel as a host list through the streamed decode kernels (12 x 4 row parts fill the
+    down kernel's lanes), 20 handles build a device table for the general kernels; a handle may
+    appear twice; routes are a strided view read through slots."""
+    announce("grouped full shape", fmt, count)
+    d, f = 2048, 512
+    hosts, dev = handles((fmt, fmt, fmt), cuda, d=d, f=f, count=min(count, 6), seed=10900)
+    order = [i % len(dev) for i in range(count)]
+    scale = np.float32(1.0 if fmt in ("Q8_0", "Q6_K") else 2.0 ** -6)
+    x = np.random.default_rng(109).normal(0, 2, (1, d)).astype(np.float32) * scale
+    routes_host = np.random.default_rng(110).normal(0, 1, count).astype(np.float32)
+    slots = tuple(int(i) for i in np.random.default_rng(111).permutation(count))
+    selected = [tuple(triple(w) for w in hosts[i]) for i in order]
+    want = R.grouped_decode(x, selected, routes_host, slots)
+    xd = torch.from_numpy(x).to(cuda)
+    routes = torch.from_numpy(np.repeat(routes_host, 3)).to(cuda)[::3]   # strided view
+    got = grouped_quantized_experts_forward(xd, [dev[i] for i in order], routes, routing_slots=slots)
+    assert got.shape == (1, d) and got.dtype == torch.float32
+    assert rel_l2(got.cpu().numpy(), want) <= 2e-5 <= REL_L2
+    again = grouped_quantized_experts_forward(xd, [dev[i] for i in order], routes, routing_slots=slots)
+    assert torch.equal(got, again) and got.data_ptr() != again.data_ptr()   # fresh output, reused scratch
+
+
 @pytest.mark.parametrize("case,reason", [
     ("batch", "contiguous"), ("noncontiguous", "contiguous"), ("dtype", "FP32"),
     ("routes_shape", "routing_weights"), ("routes_dtype", "routing_weights"),
