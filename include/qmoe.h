@@ -258,7 +258,9 @@ int qmoe_routing_plan(const int64_t* ids, const float* weights, int tokens, int 
  * 2048 / 512 / 2048 fits up to 64 tokens).  The call allocates nothing, clears nothing and
  * does not synchronise.  All calls on one GPU share the one array, which keeps the last call's
  * contents: calls that overlap on one GPU (different streams, or threads) race and must be
- * serialised by the caller; calls on one stream are ordered by the stream. */
+ * serialised by the caller; calls on one stream are ordered by the stream.  The array's address on
+ * a device is looked up once, by qmoe_init or by the first call on that device: callers that record
+ * a HIP graph call qmoe_init first, because that look-up is not stream work. */
 #define QMOE_MOE_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
 size_t qmoe_moe_static_scratch_bytes(void);
 int qmoe_moe_forward_static(const qmoe_moe_args* args, void* stream);

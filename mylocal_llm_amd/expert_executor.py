@@ -3,7 +3,8 @@
 The reference's ``ExpertsInference`` (mini_llm/ops/experts_inference.py:160-312) talks to a
 ``HeterogeneousExpertExecutor`` (mini_llm/ops/expert_residency.py:797-819) through a small set of
 hooks: ``try_forward_device_plan`` for one token (:1025-1030), ``dispatch_scope`` around a layer's
-launches (:539-560), ``try_forward_grouped`` for the singleton decode plan (:1166-1193) and
+launches (:539-560), ``try_forward_grouped`` for the singleton decode plan (:1166-1193),
+``try_forward_decode_batch`` for the same plan inside a dispatch scope (:1032-1068) and
 ``forward(layer, expert, x)`` for one expert.  That executor exists to juggle a device cache, host
 copies and CPU workers for a model that does not fit the GPU.  On a part with 288 GB of HBM every
 expert of every layer stays on the device, so this executor keeps one ``DevicePackedExpertBank``
@@ -119,6 +120,27 @@ class ResidentExpertExecutor:
         self.counters["gpu_experts"] += len(experts)
         self.counters["grouped_gpu_dispatches"] += 1
         return grouped_quantized_experts_forward(x, experts, routing_weights, routing_slots=slots)
+
+    def try_forward_decode_batch(self, layer_id, expert_ids, x, routing_weights, slots, *, on_cpu_submitted=None):
+        """Singleton decode inside a dispatch scope: unique ascending ``expert_ids`` share one fp32
+        activation (mini_llm/ops/expert_residency.py:1032-1068).  The reference shares that
+        activation across CPU misses and takes the grouped device path when every expert is already
+        admitted; here every expert always is, so the call is that grouped path.  Declines (None) what
+        the reference declines: outside a dispatch scope, another shape or dtype, ids that are not
+        unique and ascending."""
+        if (not self._dispatch_depth or tuple(x.shape) != (1, self.d_model) or x.dtype != torch.float32
+                or routing_weights.dtype != torch.float32):
+            return None
+        expert_ids = tuple(int(e) for e in expert_ids)
+        if not expert_ids or expert_ids != tuple(sorted(set(expert_ids))):
+            return None
+        output = self.try_forward_grouped(layer_id, expert_ids, x, routing_weights, tuple(slots))
+        if output is None:
+            return None
+        self.counters["admission_grouped_dispatches"] += 1
+        if on_cpu_submitted is not None:
+            on_cpu_submitted()
+        return output
 
     def stats(self):
         return {"layers": len(self.banks), "resident_bytes": self.resident_bytes, **self.counters}

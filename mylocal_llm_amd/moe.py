@@ -171,6 +171,10 @@ def router_logits(x, router_weight, router_bias=None):
     e = router_weight.shape[0]
     if router_bias is not None and (router_bias.dtype != torch.float32 or tuple(router_bias.shape) != (e,) or router_bias.device != x.device):
         raise ValueError("router_bias must be CUDA float32 [E]")
+    if d % 4 or x.data_ptr() % 16 or router_weight.data_ptr() % 16:
+        # outside what the kernel reads with 16-byte loads: the plain fp32 product, as the reference computes it
+        out = x @ router_weight.t()
+        return out if router_bias is None else out + router_bias
     logits = torch.empty((t, e), dtype=torch.float32, device=x.device)
     if t:
         with torch.cuda.device(x.device):
@@ -407,12 +411,13 @@ class Qwen3NextMoEInference:
             raise ValueError('hidden must have shape [positive batch,time,d_model]')
         if not residual.shape[1]:
             return residual.clone()
+        rows, bias = self.router.rows_and_bias()   # (whatever the router holds now, bias included)
         if self.shared_is_dense:
-            normalized, _ = norm_router(residual.reshape(-1, residual.shape[-1]).contiguous(), gamma, eps, self._router_weight)
+            normalized, _ = norm_router(residual.reshape(-1, residual.shape[-1]).contiguous(), gamma, eps, rows, bias)
             return residual + self.forward(normalized.reshape(residual.shape))
         b, t, d = residual.shape
         flat = residual.reshape(b * t, d).contiguous()
-        normalized, logits = norm_router(flat, gamma, eps, self._router_weight)
+        normalized, logits = norm_router(flat, gamma, eps, rows, bias)
         out = moe_step(normalized, self.bank, self.top_k, logits=logits, shared=self.shared, shared_gate=self.shared_gate,
                        floor=self.router.normalization_floor, residual=flat)
         return out.reshape(b, t, d)
@@ -426,7 +431,7 @@ class Qwen3NextMoEInference:
             return torch.empty_like(hidden)
         b, t, d = hidden.shape
         flat = hidden.reshape(b * t, d).contiguous()
-        logits = router_logits(flat, self._router_weight)
+        logits = self.router.logits(flat)
         if self.shared_is_dense:
             # routed part on the packed kernels; shared expert and its admission gate as fp32
             # matmuls (mini_llm/external/gguf_projection.py:40-88, qwen3next_moe.py:145-147)

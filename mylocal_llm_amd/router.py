@@ -100,16 +100,25 @@ class RouterInference:
         weights, ids, _ = expert_topk_forward(logits, self.k, return_cache=False)
         return weights, ids
 
-    def forward(self, x):
-        batch_size, seq_len, _ = x.shape
-        from .moe import router_logits
+    def rows_and_bias(self):
+        """The router matrix as the kernels read it ([n_experts, d_model] fp32, cached until W_router
+        is replaced or written to) and the bias as fp32 (or None)."""
         w = self.W_router
         stamp = (w.data_ptr(), w._version, tuple(w.shape), w.device)
         if self._rows is None or self._rows[0] != stamp:
             self._rows = (stamp, w.to(torch.float32).t().contiguous())
-        x2 = x.reshape(batch_size * seq_len, self.d_model).to(torch.float32).contiguous()
         bias = None if self.b_router is None else self.b_router.to(torch.float32).contiguous()
-        logits = router_logits(x2, self._rows[1], bias)
+        return self._rows[1], bias
+
+    def logits(self, x2):
+        """fp32 logits [T, n_experts] of rows ``x2`` [T, d_model]."""
+        from .moe import router_logits
+        rows, bias = self.rows_and_bias()
+        return router_logits(x2.to(torch.float32).contiguous(), rows, bias)
+
+    def forward(self, x):
+        batch_size, seq_len, _ = x.shape
+        logits = self.logits(x.reshape(batch_size * seq_len, self.d_model))
         logits = logits.reshape(batch_size, seq_len, self.n_experts)
         weights, ids = self.route_logits(logits)
         return weights.to(x.dtype), ids

@@ -50,6 +50,16 @@ def test_hooks_answer_from_the_resident_bank(cuda):
         with ex.dispatch_scope(lid, (2, 5, 9)):
             grouped = ex.try_forward_grouped(lid, (2, 5, 9), xd, wd.reshape(-1), (1, 2, 0))    # slots of experts 2, 5, 9
         assert rel_l2(grouped.cpu().numpy(), want) <= 2e-5
+        # the decode-batch hook: the same plan inside a dispatch scope, None for what the reference declines
+        assert ex.try_forward_decode_batch(lid, (2, 5, 9), xd, wd.reshape(-1), (1, 2, 0)) is None          # no scope
+        with ex.dispatch_scope(lid, (2, 5, 9)):
+            seen = []
+            batched = ex.try_forward_decode_batch(lid, (2, 5, 9), xd, wd.reshape(-1), (1, 2, 0), on_cpu_submitted=lambda: seen.append(1))
+            assert seen == [1] and torch.equal(batched, grouped)
+            assert ex.try_forward_decode_batch(lid, (5, 2, 9), xd, wd.reshape(-1), (2, 1, 0)) is None      # not ascending
+            assert ex.try_forward_decode_batch(lid, (2, 2, 9), xd, wd.reshape(-1), (1, 1, 0)) is None      # not unique
+            assert ex.try_forward_decode_batch(lid, (2, 5, 9), xd.half(), wd.reshape(-1), (1, 2, 0)) is None
+            assert ex.try_forward_decode_batch(lid, (), xd, wd.reshape(-1), ()) is None
         # several tokens in one step
         xn = rng.standard_normal((6, d)).astype(np.float32)
         idn = np.stack([rng.permutation(e)[:k] for _ in range(6)]).astype(np.int64)

@@ -84,3 +84,43 @@ def test_second_half_of_a_decoder_layer(cuda, tokens):
     unfused = hd + moe.forward(nd.reshape(1, tokens, d))
     assert rel_l2(got.cpu().numpy().reshape(tokens, d), unfused.cpu().numpy().reshape(tokens, d)) <= 2e-6
     assert moe.forward_after_norm(hd[:, :0], torch.from_numpy(gamma).to(cuda), 1e-6).shape == (1, 0, d)
+
+
+def test_router_bias_set_later_is_used_and_odd_widths_route(cuda):
+    """A bias written to the module's router after construction changes the routing of forward and
+    forward_after_norm (both read the router's current weight and bias); logits of rows whose width
+    is not a multiple of four come from the plain fp32 product instead of an error."""
+    from mylocal_llm_amd.moe import router_logits
+    from mylocal_llm_amd.router import RouterInference
+    announce("router bias / odd width")
+    e, d, f, fsh, k, tokens = 16, 256, 256, 512, 4, 3
+    gate, up, down, shared, gate_vec = make_layer(e, d, f, fsh, ("Q8_0", "Q8_0", "Q8_0"), 910)
+    rng = np.random.default_rng(91)
+    router_w = rng.normal(0, .3, (e, d)).astype(np.float32)
+    bias = np.zeros(e, np.float32)
+    bias[[3, 11]] = 50.0                                   # these two experts now win every row
+    hidden = rng.normal(0, 2, (1, tokens, d)).astype(np.float32)
+    moe = Qwen3NextMoEInference(DevicePackedExpertBank(gate, up, down, device=cuda), k, torch.from_numpy(router_w).to(cuda),
+                                tuple(upload(w, cuda) for w in shared), torch.from_numpy(gate_vec).to(cuda))
+    hd = torch.from_numpy(hidden).to(cuda)
+    before = moe.forward(hd)
+    moe.router.b_router = torch.from_numpy(bias).to(cuda)
+    after = moe.forward(hd)
+    flat = hidden.reshape(tokens, d)
+    logits = R.router_logits(flat, router_w, bias)
+    assert not synthetic.has_topk_ties(logits, k)
+    want, _, ids = oracle_step(flat, logits, k, gate, up, down, shared, gate_vec)
+    assert {3, 11} <= set(ids[0].tolist())
+    assert rel_l2(after.reshape(tokens, d).cpu().numpy(), want) <= 2e-5
+    assert rel_l2(before.reshape(tokens, d).cpu().numpy(), want) > 1e-3
+    # odd width: d_model = 6
+    r = RouterInference(6, 5, 2)
+    r.W_router = torch.from_numpy(rng.normal(0, 1, (6, 5)).astype(np.float32)).to(cuda)
+    r.b_router = torch.from_numpy(rng.normal(0, 1, 5).astype(np.float32)).to(cuda)
+    x = torch.from_numpy(rng.normal(0, 1, (2, 3, 6)).astype(np.float32)).to(cuda)
+    w, ids = r.forward(x)
+    want_logits = x.reshape(6, 6).cpu().numpy() @ r.W_router.cpu().numpy() + r.b_router.cpu().numpy()
+    want_w, want_ids = R.router_topk(want_logits, 2, renormalize=False)
+    np.testing.assert_array_equal(ids.reshape(6, 2).cpu().numpy(), want_ids)
+    np.testing.assert_allclose(w.reshape(6, 2).cpu().numpy(), want_w, rtol=2e-6, atol=2e-7)
+    assert router_logits(x.reshape(6, 6).contiguous(), r.W_router.t().contiguous()).shape == (6, 5)

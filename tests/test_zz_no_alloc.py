@@ -53,9 +53,15 @@ def test_static_scratch_step_equals_workspace_step(cuda, fmt):
         a = _args(hidden, logits, bank, shared, gate_vec, want, k, 0, 0)
         assert lib.qmoe_moe_forward(ctypes.byref(a), ctypes.c_void_p(workspace.data_ptr()), nbytes, stream) == 0
         b = _args(hidden, logits, bank, shared, gate_vec, got, k, 0, 0)
+        # the device variables' addresses are resolved ahead of the call (qmoe_init), so the call itself
+        # neither allocates nor looks anything up: device memory in use is the same before and after
+        assert lib.qmoe_init() == 0
+        torch.cuda.synchronize()
+        held, free_before = torch.cuda.memory_allocated(cuda), torch.cuda.mem_get_info(cuda)[0]
         rc = lib.qmoe_moe_forward_static(ctypes.byref(b), stream)
         assert rc == 0, lib.qmoe_last_error().decode()
         torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated(cuda) == held and torch.cuda.mem_get_info(cuda)[0] == free_before
         assert np.array_equal(got.cpu().numpy().view(np.uint32), want.cpu().numpy().view(np.uint32))
 
 
