@@ -21,8 +21,10 @@
 //                   rounded, then added) and finally shared * sigmoid.
 //
 // The kernels' waits are counted by hand (s_waitcnt vmcnt with the number of newer requests), so
-// every global load in them is either a DMA or an inline-assembly load whose result is not
-// touched before the wait that covers it; stores only make those waits conservative.
+// while requests are in flight every fetch is a DMA into LDS: a load into registers that the
+// compiler can see makes it wait for everything outstanding, and one it cannot see (inline
+// assembly) is unsafe as soon as its result is copied or merged at a branch before the data has
+// arrived.  Stores only make the counted waits conservative.
 #include "qmoe_decode.hpp"
 #include "qmoe_rowdot.hpp"
 #include "qmoe_span.hpp"
@@ -69,27 +71,6 @@ __device__ __forceinline__ void dma16_at_masked(const uint8_t* lane_address, uin
     asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
                  : "=&s"(save) : "v"(lane_address), "s"(mask) : "memory");
 }
-// One dword per lane; the result must not be touched before a wait that covers the load
-// (settle() names the values such a wait has released).
-__device__ __forceinline__ uint32_t load_u32_unwaited(const void* lane_address) {
-    uint32_t v;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(lane_address) : "memory");
-    return v;
-}
-__device__ __forceinline__ void settle(uint32_t& a) { asm volatile("" : "+v"(a)::"memory"); }
-__device__ __forceinline__ u32x2_t load_u32x2_unwaited(const void* lane_address) {
-    u32x2_t v;
-    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(v) : "v"(lane_address) : "memory");
-    return v;
-}
-__device__ __forceinline__ u32x4_t load_u32x4_unwaited(const void* lane_address) {
-    u32x4_t v;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(lane_address) : "memory");
-    return v;
-}
-__device__ __forceinline__ void settle(u32x2_t& a) { asm volatile("" : "+v"(a)::"memory"); }
-__device__ __forceinline__ void settle(u32x4_t& a) { asm volatile("" : "+v"(a)::"memory"); }
-
 // s_waitcnt vmcnt(n) for a wave-uniform n known only at run time (the count is an immediate).
 __device__ __forceinline__ void wait_vmcnt_rt(int n) {
     switch (n) {
