@@ -16,7 +16,8 @@ The JSON line also carries
                 call, fp32 matmul) timed on this box's host cores on bounded samples, with the
                 library's scalar C++ host twin, configs[0] and one MoE decode token as legs
   extras        other configurations measured the same way: the layer launched in data-flow
-                order, other formats and token counts, MoE decode (cold rotation, and hot)
+                order, other formats and token counts, MoE decode (cold rotation, and hot), the
+                grouped decode call, the layer half, MoE prefill, the vocabulary projection
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
 """
@@ -506,6 +507,45 @@ def layer_extra(torch, lib, device, fmt, tokens, act, steps, by_dependency=False
     return out
 
 
+def vocabulary_projection_extra(torch, lib, device, fmt, steps, copies=2):
+    """The output projection of the reference's model at its real shape (151 936 x 2048,
+    mini_llm/external/qwen3next_model.py:291-293), one token, one qmoe_linear call per step;
+    steps alternate between `copies` matrices (each larger than the memory-side cache)."""
+    from mylocal_llm_amd import _lib
+    n, k = 151936, 2048
+    gen = torch.Generator(device=device)
+    gen.manual_seed(606)
+    weights = [device_blocks(torch, fmt, n, k, gen, device) for _ in range(copies)]
+    x = torch.randn((1, k), device=device, generator=gen)
+    y = torch.empty((1, n), device=device, dtype=torch.float32)
+    fid, turn = _lib.FORMAT_ID[fmt], [0]
+
+    def step(stream):
+        w = weights[turn[0] % copies]
+        turn[0] += 1
+        rc = lib.qmoe_linear(w.data_ptr(), fid, n, k, x.data_ptr(), 0, 1, y.data_ptr(), 0, stream)
+        if rc:
+            raise RuntimeError(lib.qmoe_last_error().decode())
+
+    _, ms = time_steps(torch, step, steps, 2)
+    per_call = ms / steps * 1e-3
+    nbytes = weight_bytes(fmt, n, k)
+    out = {"workload": f"vocabulary projection {fmt} 151936x2048 M=1", "weight_bytes": nbytes,
+           "us_per_call": round(per_call * 1e6, 2), "GBps": round(nbytes / per_call / 1e9, 1),
+           "frac_hbm_peak": round(nbytes / per_call / 1e9 / HBM_PEAK_GBS, 4)}
+    del weights
+    torch.cuda.empty_cache()
+    return out
+
+
+def guarded(fn, *args, **kwargs):
+    """An extras entry, or the reason it could not be measured (the headline line is printed either way)."""
+    try:
+        return fn(*args, **kwargs)
+    except Exception as exc:   # noqa: BLE001 - the message goes into the JSON line
+        return {"workload": getattr(fn, "__name__", "extra"), "error": f"{type(exc).__name__}: {exc}"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -514,7 +554,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_timeline", "moe_layer_half", "grouped_decode", "layer_few_tokens", "read_probe",
+    ap.add_argument("--only", choices=["moe_prefill", "moe_decode", "moe_decode_hot", "moe_timeline", "moe_layer_half", "grouped_decode", "layer_few_tokens", "read_probe", "vocabulary_projection",
                                        "layer_q6_k", "layer_q5_k", "layer_q4_k", "layer_by_dependency"], default=None,
                     help="run one of the extra workloads alone and print its JSON (profiling runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -558,6 +598,9 @@ def main():
         return
     if args.only == "layer_by_dependency":
         print(json.dumps(layer_extra(torch, lib, device, "Q8_0", 1, "f32", max(10, args.steps), by_dependency=True)))
+        return
+    if args.only == "vocabulary_projection":
+        print(json.dumps([vocabulary_projection_extra(torch, lib, device, fmt, max(10, args.steps)) for fmt in ("Q8_0", "Q6_K")]))
         return
     if args.only == "moe_layer_half":
         print(json.dumps([moe_decode_extra(torch, lib, device, "Q8_0", t, max(8, args.steps), args.warmup, layer_half=True) for t in (1, 4)]))
@@ -628,6 +671,8 @@ def main():
         for fmt in ("Q8_0", "Q6_K", "Q5_K"):
             extras.append(moe_prefill_extra(torch, lib, device, fmt, 512, 6, 2))
             torch.cuda.empty_cache()
+        for fmt in ("Q8_0", "Q6_K"):
+            extras.append(guarded(vocabulary_projection_extra, torch, lib, device, fmt, max(10, args.steps)))
         result["extras"] = extras
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
