@@ -151,3 +151,56 @@ def test_product_package_never_imports_the_oracle():
             if name.endswith((".py", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(base, name)).read()
                 assert "oracle" not in text.replace("no oracle", ""), os.path.join(base, name)
+
+
+@pytest.mark.parametrize("tokens,n_experts,k", [(2500, 512, 10), (1900, 512, 1), (929, 512, 4), (70000, 8, 2)])
+def test_routing_plan_of_token_chunks_is_the_plan_of_the_whole_batch(tokens, n_experts, k, monkeypatch):
+    """Batches beyond what one plan-kernel call covers are planned in token chunks and joined with
+    index arithmetic: with the kernel call replaced by the oracle's plan of each chunk (host tensors),
+    the joined plan must be the oracle's plan of the whole batch, Zipf-skewed routing included."""
+    import torch
+    from oracle import reference_np as R
+    from mylocal_llm_amd import routing_plan as rp, synthetic
+
+    calls = []
+
+    def oracle_call(ids, w, kk, e):
+        n = ids.shape[0]
+        calls.append(n)
+        assert n <= min(512, rp.max_tokens_per_plan_call(e)) and ids.is_contiguous() and w.is_contiguous()
+        token, _, order, offsets = R.routing_plan(ids.numpy(), e)
+        pos = np.empty(n * kk, dtype=np.int32)
+        pos[order] = np.arange(n * kk, dtype=np.int32)
+        as_i32 = lambda a: torch.from_numpy(np.asarray(a, dtype=np.int32))
+        return (as_i32(offsets), as_i32(order), as_i32(token), torch.from_numpy(w.numpy().reshape(-1)[order].copy()),
+                torch.from_numpy(pos), torch.zeros(1, dtype=torch.int32))
+
+    logits = synthetic.router_logits(tokens, n_experts, 5, zipf=1.1)
+    w, ids = R.router_topk(logits, k, floor=2.0 ** -14)
+    plan = rp.RoutingPlan._build(torch.from_numpy(ids.reshape(1, tokens, k)), torch.from_numpy(w.reshape(1, tokens, k)), k, n_experts, oracle_call)
+    assert len(calls) == -(-tokens // 512) > 1 and sum(calls) == tokens
+    token, slot, order, offsets = R.routing_plan(ids, n_experts)
+    assert plan.expert_offsets == tuple(int(v) for v in offsets)
+    np.testing.assert_array_equal(plan.order.numpy(), order)
+    np.testing.assert_array_equal(plan.token_indices.numpy(), token)
+    np.testing.assert_array_equal(plan.slot_indices.numpy(), slot)
+    np.testing.assert_array_equal(plan.expert_indices.numpy(), ids.reshape(-1)[order])
+    np.testing.assert_array_equal(plan.weights.numpy(), w.reshape(-1)[order])
+    np.testing.assert_array_equal(order[plan.position_of_assignment.numpy().reshape(-1)], np.arange(tokens * k))
+    assert plan.active_expert_ids() == tuple(int(i) for i in np.nonzero(np.bincount(ids.reshape(-1), minlength=n_experts))[0])
+
+
+def test_routing_plan_of_token_chunks_reports_invalid_routing(monkeypatch):
+    """A chunk whose plan is flagged (and may hold anything) makes the joined plan raise; no look-up
+    of the join leaves its arrays on the way."""
+    import torch
+    from mylocal_llm_amd import routing_plan as rp
+
+    def flagged(ids, w, kk, e):
+        n = ids.shape[0] * kk
+        junk = torch.full((n,), 2 ** 31 - 1, dtype=torch.int32)
+        return (torch.zeros(e + 1, dtype=torch.int32), junk, junk.clone(), torch.zeros(n), -junk, torch.ones(1, dtype=torch.int32))
+
+    ids = torch.zeros((1, 2000, 2), dtype=torch.int64)
+    with pytest.raises(ValueError, match="Invalid routing"):
+        rp.RoutingPlan._build(ids, torch.zeros((1, 2000, 2)), 2, 512, flagged)
