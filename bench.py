@@ -209,6 +209,24 @@ def cpu_baseline(budget_s=24.0):
     legs.append({"workload": "MoE decode T=1 (512 experts, top-10, D=2048, F=512, shared 2048), NumPy", "cores": int(threads),
                  "kind": "port", "GBps": round(moe_bytes / moe_s / 1e9, 4), "ms": round(moe_s * 1e3, 2),
                  "tokens_per_s": round(1.0 / moe_s, 3), "repetitions": 1})
+    # the reference's opt-in native backend (cpu_packed_backend="native"): its own native_packed_cpu.cpp,
+    # compiled by oracle/Makefile with the flags the reference itself uses, where that build is present
+    try:
+        from oracle import native as oracle_native
+        if oracle_native.load_ref() is not None:
+            ref_s = {}
+            for shape, w in distinct.items():
+                oracle_native.ref_gemv(xs[shape[1]], w.data, w.shape, "Q8_0")   # untimed
+                t0 = time.perf_counter()
+                oracle_native.ref_gemv(xs[shape[1]], w.data, w.shape, "Q8_0")
+                ref_s[shape] = time.perf_counter() - t0
+            ref_layer_s = sum(ref_s[shape] for shape in shapes)
+            legs.append({"workload": "one 8B layer, Q8_0, M=1, all seven projections: the reference's own native_packed_cpu.cpp "
+                                     "(mylocal_packed_gemv, g++ -O3 as the reference builds it; oracle/_ref)",
+                         "cores": 1, "kind": "reference", "GBps": round(layer_bytes / ref_layer_s / 1e9, 4),
+                         "ms": round(ref_layer_s * 1e3, 2), "tokens_per_s_32_layers": round(1.0 / (32 * ref_layer_s), 4), "repetitions": 1})
+    except Exception as exc:   # noqa: BLE001 - a missing or unloadable build only drops this leg
+        legs.append({"workload": "the reference's native_packed_cpu.cpp (oracle/_ref)", "error": f"{type(exc).__name__}: {exc}"})
     return {"value": round(layer_bytes / layer_s / 1e9, 4), "unit": "GB/s", "cores": int(threads), "kind": "port",
             "sample": f"one 8B layer, Q8_0, M=1: all seven projections ({layer_bytes} weight bytes) multiplied once each "
                       f"(one warm-up and one timed call per distinct shape, {layer_s:.2f}s per layer), NumPy dequantise-every-call + fp32 matmul "
