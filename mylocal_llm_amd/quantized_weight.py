@@ -113,10 +113,6 @@ class PackedGGUFWeight:
         return self._view(start * self._row_bytes, (stop - start, self.shape[1]))
 
     # ---- the reference's host helpers, on the library's host twins -----------------------------
-    @staticmethod
-    def _reference_tile_rows(tile_rows):
-        return _positive_int(tile_rows, "tile_rows must be a positive integer")
-
     def _decode_rows(self, raw, rows):
         """fp32 [rows, columns] of ``rows`` packed rows lying contiguously in ``raw``."""
         from . import _lib
@@ -137,7 +133,7 @@ class PackedGGUFWeight:
         only the requested rows are decoded, ``tile_rows`` of them at a time."""
         if len(self.shape) != 2:
             raise ValueError("selected rows require a matrix; select_outer first")
-        step = self._reference_tile_rows(tile_rows)
+        step = _positive_int(tile_rows, "tile_rows must be a positive integer")
         wanted = np.asarray(indices)
         if wanted.ndim != 1 or wanted.dtype.kind not in "iu":
             raise ValueError("indices must be a one-dimensional integer array")
@@ -156,7 +152,7 @@ class PackedGGUFWeight:
         validated as in the reference (the host linear walks row by row and needs no tiling)."""
         if len(self.shape) != 2:
             raise ValueError("matvec requires a matrix; select_outer first")
-        self._reference_tile_rows(tile_rows)
+        _positive_int(tile_rows, "tile_rows must be a positive integer")
         vector = np.asarray(vector, dtype=np.float32)
         if vector.shape != (self.shape[1],):
             raise ValueError("vector shape must equal (matrix columns,)")
