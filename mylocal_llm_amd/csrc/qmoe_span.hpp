@@ -33,6 +33,15 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 // outstanding requests of a load it knows to write LDS; the waits are this file's own.
 #define QMOE_DMA16(base, voff, OFFSET) \
     asm volatile("global_load_lds_dwordx4 %0, %1 offset:" #OFFSET :: "v"(voff), "s"(uniform((const uint8_t*)(base))) : "memory")
+// (Two wait-state rules of the ISA manual that the compiler keeps for its own instructions are NOT
+// kept around this inline assembly, which its hazard recogniser does not look into: one wait state
+// between a scalar write of M0 and an LDS-DMA that reads it (back to back in the whole-slot request
+// of span_kernel), and five between a vector instruction that writes a scalar register
+// (v_readfirstlane, what uniform() becomes when the value lives in vector registers: the base of a
+// gate/up pair's request) and a memory instruction that reads it as its base.  Every result of
+// those requests has been right on MI355X, where the hardware evidently settles both; the
+// by-the-book form is an "s_nop 0" behind the s_mov below and an "s_nop 4" ahead of a load whose
+// base was just made uniform, at the price of issue slots in the streaming loop.)
 __device__ __forceinline__ void set_m0(uint32_t v) { asm volatile("s_mov_b32 m0, %0" :: "s"(uniform((int)v)) : "memory"); }
 // the same on the lanes of `mask` only (a wave-uniform 64-bit lane mask, not zero)
 __device__ __forceinline__ void dma16_masked(const void* base, uint32_t voff, uint64_t mask) {
