@@ -119,6 +119,40 @@ def test_invalid_arguments_return_codes_before_any_launch():
     assert lib.qmoe_moe_forward(None, null, 0, null) == 1
 
 
+def test_listed_grouped_decode_rejects_bad_arguments_before_any_launch():
+    """qmoe_grouped_decode_listed reads its expert list on the host: every rejection below happens
+    before anything is launched (no GPU needed), with the status code the header names."""
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    fake = ctypes.c_void_p(4096)
+    table = (ctypes.c_void_p * 6)(4096, 8192, 12288, 16384, 20480, 24576)
+    listed = ctypes.cast(table, ctypes.c_void_p)
+    call = lambda **kw: lib.qmoe_grouped_decode_listed(*[kw.get(name, default) for name, default in (
+        ("x", fake), ("experts", listed), ("n", 2), ("gf", 0), ("uf", 0), ("df", 0), ("d", 256), ("f", 256), ("routes", fake),
+        ("stride", 1), ("slots", null), ("out", fake), ("ws", fake), ("stream", null))])
+    assert call(x=null) == 1 and call(experts=null) == 1 and call(routes=null) == 1 and call(out=null) == 1
+    assert call(ws=null) == 4 and call(ws=ctypes.c_void_p(4100)) == 4           # workspace missing / not 16-byte aligned
+    assert b"workspace" in lib.qmoe_last_error()
+    assert call(n=0) == 1
+    assert call(n=17) == 2 and b"qmoe_grouped_decode" in lib.qmoe_last_error()    # beyond a host list: the device-table entry
+    assert call(d=0) == 1 and call(f=-256) == 1
+    assert call(gf=42) == 1 and b"unknown" in lib.qmoe_last_error()
+    assert call(d=200) == 1 and b"block multiple" in lib.qmoe_last_error()          # Q8_0: K not a multiple of 32
+    holes = (ctypes.c_void_p * 6)(4096, 0, 12288, 16384, 20480, 24576)
+    assert call(experts=ctypes.cast(holes, ctypes.c_void_p)) == 1 and b"null projection" in lib.qmoe_last_error()
+    odd = (ctypes.c_void_p * 6)(4097, 8192, 12288, 16384, 20480, 24576)
+    assert call(experts=ctypes.cast(odd, ctypes.c_void_p)) == 1 and b"2-byte aligned" in lib.qmoe_last_error()
+    negative = (ctypes.c_int32 * 2)(0, -1)
+    assert call(slots=ctypes.cast(negative, ctypes.c_void_p)) == 1 and b"route position" in lib.qmoe_last_error()
+
+
+def test_wait_limit_and_abi_version_are_plain_host_calls():
+    lib = _lib.load()
+    assert lib.qmoe_abi_version() == _lib.ABI_VERSION == 5
+    lib.qmoe_set_wait_limit(12345)     # stored for the next launches; nothing touches a device
+    lib.qmoe_set_wait_limit(0)         # back to the default
+
+
 def test_moe_workspace_size_is_monotone_and_aligned():
     lib = _lib.load()
     a = lib.qmoe_moe_workspace_bytes(1, 10, 512, 2048, 512, 2048)
