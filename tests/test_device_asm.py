@@ -58,3 +58,24 @@ def test_decode_kernels_keep_the_wait_state_behind_an_m0_write(findings):
     """No LDS-DMA of the MoE decode kernels follows its M0 write back to back."""
     offenders = {k: v["m0_back_to_back"] for k, v in findings["qmoe_decode2.hip"].items() if v["m0_back_to_back"]}
     assert not offenders, offenders
+
+
+def test_multiply_high_division_is_exact_where_the_decode_plans_allow_it():
+    """The MoE decode kernels divide item and piece numbers by run-time constants with one
+    multiply-high: q / d = (q * (floor(2^32 / d) + 1)) >> 32.  The host plans admit a launch only
+    while dividend x divisor < 2^32 (csrc/qmoe_decode2.hip: pairs2_plan, down2_plan); inside that
+    bound the quotient is exact -- checked here at the bound's edge for every divisor the plans can
+    produce and on random dividends below it."""
+    import numpy as np
+    rng = np.random.default_rng(5)
+    divisors = sorted(set(range(1, 600)) | {1024, 2048, 4096, 7168, 14336, 65536, 151936})
+    for d in divisors:
+        if d == 1:
+            continue                                  # (k == 1 is special-cased in the kernel: the magic number overflows)
+        magic = (1 << 32) // d + 1
+        assert magic < (1 << 32)
+        limit = ((1 << 32) - 1) // d                  # largest dividend with q * d < 2^32
+        q = np.unique(np.concatenate([np.arange(0, min(limit, 4096) + 1), np.arange(max(0, limit - 4096), limit + 1),
+                                      rng.integers(0, limit + 1, 4096)])).astype(np.uint64)
+        got = (q * np.uint64(magic)) >> np.uint64(32)
+        assert np.array_equal(got, q // np.uint64(d)), d
